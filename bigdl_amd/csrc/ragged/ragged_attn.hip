@@ -1,5 +1,6 @@
-// Paged attention of the ragged engine: causal sliding window that also keeps the first tokens, one or two score maps
-// per head over shared values (differential attention), per-head output norm and sigmoid gate in the epilogue.
+// Paged attention of the ragged engine: causal sliding window that also keeps the first tokens and / or a mask of blocks
+// counted from the sequence's start, soft-capped scores, one or two score maps per head over shared values
+// (differential attention), per-head output norm and sigmoid gate (per head or per channel) in the epilogue.
 //
 // paged_attn_kernel (this file): one workgroup serves one (token row, query head).  A cache page holds 64 keys, one per
 // lane, so the scores of a page are one register per map and the softmax statistics are wavefront reductions; values
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
   for (int c = threadIdx.x; c < REP * qd; c += blockDim.x) qs[c] = a.q[((int64_t)t * a.H + h0) * qd + c];
   __syncthreads();
 
-  const int lo = a.window > 0 ? (i - a.window + 1 > 0 ? i - a.window + 1 : 0) : 0;
+  const int lo_raw = low_key(i, a.window, a.chunk);
+  const int lo = lo_raw > 0 ? lo_raw : 0;
   const int keep = a.window > 0 ? a.keep_first : 0;
   const T* K = (const T*)a.kpages;
   const T* V = (const T*)a.vpages;
@@ -192,6 +194,13 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
 #pragma unroll
         for (int mp = 0; mp < MAPS; ++mp) s[r][mp] *= a.scale;
     }
+    if (a.softcap > 0.f) {
+      const float inv_cap = 1.0f / a.softcap;
+#pragma unroll
+      for (int r = 0; r < REP; ++r)
+#pragma unroll
+        for (int mp = 0; mp < MAPS; ++mp) s[r][mp] = a.softcap * tanhf(s[r][mp] * inv_cap);
+    }
     if (U < nk) load_values(vb, U);
     // softmax statistics of all heads and maps side by side (their cross-lane steps overlap)
     float p[REP][MAPS], mx[REP][MAPS], sm[REP][MAPS];
@@ -298,13 +307,19 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
     }
     float f = a.out_scale;
     if (a.out_norm) f *= 1.0f / sqrtf(wave_sum(ss) / (float)a.vd + a.eps);
-    if (a.gate) f *= sigmoidf_(to_f(((const T*)a.gate)[(int64_t)t * a.ldg + a.gate0 + h]));
+    if (a.gate && !a.gate_wide) f *= sigmoidf_(to_f(((const T*)a.gate)[(int64_t)t * a.ldg + a.gate0 + h]));
     T* orow = (T*)a.out + (int64_t)t * a.H * a.vd + (int64_t)h * a.vd;
+    const T* grow = (const T*)a.gate + (int64_t)t * a.ldg + a.gate0 + (int64_t)h * a.vd;     // (read only with gate_wide)
 #pragma unroll
     for (int v = 0; v < VRP; ++v) {
       const int c = 2 * lane + 128 * v;
-      if (c < a.vd) orow[c] = from_f<T>(o[v][0] * f);
-      if (c + 1 < a.vd) orow[c + 1] = from_f<T>(o[v][1] * f);
+      float f0 = f, f1 = f;
+      if (a.gate_wide) {
+        if (c < a.vd) f0 *= sigmoidf_(to_f(grow[c]));
+        if (c + 1 < a.vd) f1 *= sigmoidf_(to_f(grow[c + 1]));
+      }
+      if (c < a.vd) orow[c] = from_f<T>(o[v][0] * f0);
+      if (c + 1 < a.vd) orow[c + 1] = from_f<T>(o[v][1] * f1);
     }
   }
 }
@@ -317,7 +332,9 @@ static void launch_one(AttnArgs a, Batch bt, int nrows, int coal, hipStream_t st
   // as many wavefronts as a row can have visible pages (longest sequence of the batch), at most 8, fewer if the
   // partial results would not fit 48 KB of LDS
   int nw = 8;
-  const int most = a.window > 0 ? (a.window + PAGE - 1) / PAGE + 1 + (a.keep_first + PAGE - 1) / PAGE : bt.max_pages;
+  int most = bt.max_pages;
+  if (a.window > 0) most = (a.window + PAGE - 1) / PAGE + 1 + (a.keep_first + PAGE - 1) / PAGE;
+  if (a.chunk > 0 && (a.chunk + PAGE - 1) / PAGE + 1 < most) most = (a.chunk + PAGE - 1) / PAGE + 1;
   while (nw > 1 && nw / 2 >= (most < bt.max_pages ? most : bt.max_pages)) nw >>= 1;
   auto lds = [&](int w) { return (size_t)(((REP * qd + 3) & ~3) + w * wstride) * sizeof(float); };
   while (nw > 1 && lds(nw) > 48 * 1024) nw >>= 1;
@@ -354,7 +371,7 @@ static void launch_rows(AttnArgs a, Batch bt, int nrows, hipStream_t st, int* rc
 
 extern "C" int ragged_paged_attn(AttnArgs a, Batch bt, int maps, int dtype, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || a.d <= 0 || a.vd <= 0 || a.vd > 128 * MAX_VRP) return -1;
-  if ((maps != 1 && maps != 2) || a.ldv < a.vd) return -1;
+  if ((maps != 1 && maps != 2) || a.ldv < a.vd || a.chunk < 0 || (a.gate_wide && !a.gate)) return -1;
   const int nrows = a.rows ? a.n_rows : bt.T;
   if (nrows <= 0 || (int64_t)nrows * a.H > 0x7fffffff) return -1;
   int rc = 0;

@@ -33,6 +33,9 @@ union Frag {
 };
 
 __device__ __forceinline__ uint16_t bf_bits(float f) { return from_f<bf16>(f).b; }
+// tanh through one exponential: 1 - 2 / (e^(2x) + 1); absolute error of a few 1e-7, no overflow trouble (e^(2x) = inf
+// gives 1, 0 gives -1)
+__device__ __forceinline__ float fast_tanh(float x) { return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f); }
 
 template <int MAPS, int DK>
 __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch bt) {
@@ -68,17 +71,20 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
     }
 
   const int p_first = past + row0, p_last = past + row0 + nrows - 1;
-  const bool win = a.window > 0;
-  const int keep = win ? a.keep_first : 0;
-  const int lo_tile = win ? (p_first - a.window + 1 > 0 ? p_first - a.window + 1 : 0) : 0;
+  const bool win = a.window > 0 || a.chunk > 0;              // some keys at or below a row's position are hidden
+  const int keep = a.window > 0 ? a.keep_first : 0;
+  const int lo_first = low_key(p_first, a.window, a.chunk);
+  const int lo_tile = lo_first > 0 ? lo_first : 0;
   const int pl = lo_tile / PAGE, last = p_last / PAGE;
   const int kept_pages = (keep + PAGE - 1) / PAGE < pl ? (keep + PAGE - 1) / PAGE : pl;
   const int npg = kept_pages + last - pl + 1;
   // what this wavefront's 16 rows can see
   const int w_first = p_first + 16 * wave, w_last = (w_first + 15 < p_last ? w_first + 15 : p_last);
-  const int w_lo = win ? w_first - a.window + 1 : 0;
+  const int w_lo = low_key(w_first, a.window, a.chunk);      // (the lowest key a row sees never falls as positions grow)
+  const int w_lo_last = low_key(w_last, a.window, a.chunk);
   const bool wave_has_rows = 16 * wave < nrows;
-  const int my_lo = win ? qpos - a.window + 1 : 0;
+  const int my_lo = low_key(qpos, a.window, a.chunk);
+  const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
 
   const bf16* K = (const bf16*)a.kpages;
   const bf16* V = (const bf16*)a.vpages;
@@ -171,7 +177,7 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
     // ---- mask, online softmax (per-lane scalars of the lane's query), exponentials as two bfloat16 terms
     Frag phi[MAPS][2], plo[MAPS][2];
     // a page whose 64 keys every row of this wavefront sees needs no mask arithmetic
-    const bool inner = k0 + PAGE - 1 <= w_first && (!win || k0 >= w_last - a.window + 1 || k0 + PAGE - 1 < keep);
+    const bool inner = k0 + PAGE - 1 <= w_first && (!win || k0 >= w_lo_last || k0 + PAGE - 1 < keep);
 #pragma unroll
     for (int mp = 0; mp < MAPS; ++mp) {
       float mx = -1e30f;
@@ -181,6 +187,7 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             S[mp][kb][i] *= a.scale;
+            if (a.softcap > 0.f) S[mp][kb][i] = a.softcap * fast_tanh(S[mp][kb][i] * inv_cap);
             mx = fmaxf(mx, S[mp][kb][i]);
           }
       } else {
@@ -190,7 +197,9 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
           for (int i = 0; i < 4; ++i) {
             const int key = k0 + 16 * kb + 4 * g4 + i;
             const bool vis = key <= qpos && (key >= my_lo || key < keep);
-            S[mp][kb][i] = vis ? S[mp][kb][i] * a.scale : -1e30f;
+            float sc = S[mp][kb][i] * a.scale;
+            if (a.softcap > 0.f) sc = a.softcap * fast_tanh(sc * inv_cap);
+            S[mp][kb][i] = vis ? sc : -1e30f;
             mx = fmaxf(mx, S[mp][kb][i]);
           }
       }
@@ -267,11 +276,18 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   ss += __shfl_xor(ss, 32, 64);
   float f = a.out_scale;
   if (a.out_norm) f *= 1.0f / sqrtf(ss / (float)a.vd + a.eps);
-  if (a.gate) f *= sigmoidf_(to_f(((const bf16*)a.gate)[t * a.ldg + a.gate0 + h]));
+  if (a.gate && !a.gate_wide) f *= sigmoidf_(to_f(((const bf16*)a.gate)[t * a.ldg + a.gate0 + h]));
   uint16_t* orow = (uint16_t*)a.out + t * (int64_t)(a.H * a.vd) + (int64_t)h * a.vd;
+  const bf16* grow = (const bf16*)a.gate + t * a.ldg + a.gate0 + (int64_t)h * a.vd;        // (read only with gate_wide)
 #pragma unroll
   for (int eb = 0; eb < MF_NEB; ++eb)
     if (eb < neb) {
+      if (a.gate_wide) {                                     // one gate per channel: 8 bytes of logits per lane and block
+        Frag gl;
+        gl.d2[0] = *reinterpret_cast<const uint2*>(grow + 16 * eb + 4 * g4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) O[0][eb][i] *= sigmoidf_(__uint_as_float((uint32_t)gl.h[i] << 16));
+      }
       uint2 w;
       w.x = (uint32_t)bf_bits(O[0][eb][0] * f) | ((uint32_t)bf_bits(O[0][eb][1] * f) << 16);
       w.y = (uint32_t)bf_bits(O[0][eb][2] * f) | ((uint32_t)bf_bits(O[0][eb][3] * f) << 16);
@@ -488,7 +504,7 @@ static int launch_wide(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
 
 extern "C" int ragged_paged_attn_mfma_wide(AttnArgs a, Batch bt, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_wide_ok(a.d, a.vd)) return -1;
-  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate) return -1;
+  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate || a.chunk > 0 || a.softcap > 0.f) return -1;
   if (!a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
   const unsigned grid = (unsigned)(a.n_tiles * a.H);
   const int dk = (a.d + 31) / 32, neb = a.vd / 16;
@@ -684,7 +700,7 @@ static int launch_heads(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
 // token rows a.rows[0 .. n_rows) (all T rows without a list)
 extern "C" int ragged_paged_attn_mfma_heads(AttnArgs a, Batch bt, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_wide_ok(a.d, a.vd)) return -1;
-  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate) return -1;
+  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate || a.chunk > 0 || a.softcap > 0.f) return -1;
   const int nrows = a.rows ? a.n_rows : bt.T;
   const int nblk = (a.H / a.G + 15) / 16;
   if (nrows <= 0 || (int64_t)nrows * a.G * nblk > 0x7fffffff) return -1;
@@ -717,6 +733,8 @@ static void launch_mfma(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
 extern "C" int ragged_paged_attn_mfma(AttnArgs a, Batch bt, int maps, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_ok(a.d, a.vd)) return -1;
   if (a.ldv < a.vd || a.ldv % 8) return -1;                  // value rows are read 16 bytes at a time
+  // per-channel gate logits are read 8 bytes at a time
+  if (a.chunk < 0 || (a.gate_wide && (!a.gate || a.ldg % 4 || a.gate0 % 4))) return -1;
   if ((maps != 1 && maps != 2) || !a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
   const unsigned grid = (unsigned)(a.n_tiles * a.H);
   if (maps == 2) launch_mfma<2>(a, bt, grid, st);

@@ -9,14 +9,15 @@ using namespace ragged;
 constexpr int MOE_MAX_E = 512;      // experts
 constexpr int MOE_SLOTS = MOE_MAX_E / 64;
 
-// Scores s = softmax(W_r x) over all experts in float (x may be the bfloat16 rounding of the normed stream).  Experts
-// form `groups` equal runs of neighbours; a group's score is its best expert's; the `top` best experts of the `keep` best
-// groups are chosen, best first, with weight s * scale (no renormalisation).  Ties go to the lower lane.
+// Scores s = softmax(W_r x) over all experts (score_fn 0) or sigmoid(W_r x) per expert (score_fn 1), in float (x may be
+// the bfloat16 rounding of the normed stream).  Experts form `groups` equal runs of neighbours; a group's score is the sum
+// of its `group_top` (1 or 2) best experts' scores; the `top` best experts of the `keep` best groups are chosen, best
+// first, with weight s * scale, or (renorm) s / (sum of the chosen s + 1e-20) * scale.  Ties go to the lower lane.
 // One workgroup of four wavefronts per row: the wavefronts share the router's rows, wavefront 0 chooses.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, int64_t ldx, const float* __restrict__ wr,
                                                         int* __restrict__ idx, float* __restrict__ wts, int D, int E, int groups,
-                                                        int keep, int top, float scale) {
+                                                        int keep, int top, float scale, int score_fn, int group_top, int renorm) {
   __shared__ float z[MOE_MAX_E];
   __shared__ float gbest[64];
   extern __shared__ __attribute__((aligned(16))) float xs[];       // the row as floats
@@ -58,34 +59,50 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
   __syncthreads();
   if (wave != 0) return;
   float s[MOE_SLOTS];
-  float mx = -1e30f;
+  if (score_fn == 1) {
 #pragma unroll
-  for (int k = 0; k < MOE_SLOTS; ++k) {
-    const int e = lane + 64 * k;
-    s[k] = e < E ? z[e] : -1e30f;
-    mx = fmaxf(mx, s[k]);
-  }
-  mx = wave_max(mx);
-  float sum = 0.f;
+    for (int k = 0; k < MOE_SLOTS; ++k) {
+      const int e = lane + 64 * k;
+      s[k] = e < E ? 1.0f / (1.0f + expf(-z[e])) : 0.f;
+      if (e < E) z[e] = s[k];
+    }
+  } else {
+    float mx = -1e30f;
 #pragma unroll
-  for (int k = 0; k < MOE_SLOTS; ++k) {
-    const int e = lane + 64 * k;
-    s[k] = e < E ? expf(s[k] - mx) : 0.f;
-    sum += s[k];
-  }
-  sum = wave_sum(sum);
+    for (int k = 0; k < MOE_SLOTS; ++k) {
+      const int e = lane + 64 * k;
+      s[k] = e < E ? z[e] : -1e30f;
+      mx = fmaxf(mx, s[k]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
 #pragma unroll
-  for (int k = 0; k < MOE_SLOTS; ++k) {
-    const int e = lane + 64 * k;
-    s[k] = s[k] / sum;
-    if (e < E) z[e] = s[k];
+    for (int k = 0; k < MOE_SLOTS; ++k) {
+      const int e = lane + 64 * k;
+      s[k] = e < E ? expf(s[k] - mx) : 0.f;
+      sum += s[k];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int k = 0; k < MOE_SLOTS; ++k) {
+      const int e = lane + 64 * k;
+      s[k] = s[k] / sum;
+      if (e < E) z[e] = s[k];
+    }
   }
   // (a wavefront's LDS requests are served in order: the scores written above are what is read below)
   const int gsz = E / groups;
   if (groups > 1 && keep < groups) {
     float g = -1.f;
-    if (lane < groups)
-      for (int j = 0; j < gsz; ++j) g = fmaxf(g, z[lane * gsz + j]);
+    if (lane < groups) {
+      float second = 0.f;                                   // (scores are not negative: a group of one adds nothing)
+      for (int j = 0; j < gsz; ++j) {
+        const float v = z[lane * gsz + j];
+        if (v > g) { second = g > 0.f ? g : 0.f; g = v; }
+        else if (v > second) second = v;
+      }
+      if (group_top == 2) g += second;
+    }
     bool kept = false;
     for (int it = 0; it < keep; ++it) {
       const float best = wave_max(kept ? -1.f : g);
@@ -102,6 +119,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
 #pragma unroll
   for (int k = 0; k < MOE_SLOTS; ++k)
     if (lane + 64 * k >= E) s[k] = -1.f;
+  float total = 0.f, kept_w = 0.f;                         // lane `it` keeps the score of the it-th choice (top <= 64 with renorm)
   for (int it = 0; it < top; ++it) {
     float mine = s[0];
     int at = 0;
@@ -110,22 +128,27 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
       if (s[k] > mine) { mine = s[k]; at = k; }
     const float best = wave_max(mine);
     const unsigned long long who = __ballot(mine == best);
+    total += best;
+    if (lane == (it & 63)) kept_w = best;
     if (lane == __ffsll((long long)who) - 1) {
       idx[(int64_t)t * top + it] = lane + 64 * at;
-      wts[(int64_t)t * top + it] = best * scale;
+      if (!renorm) wts[(int64_t)t * top + it] = best * scale;
 #pragma unroll
       for (int k = 0; k < MOE_SLOTS; ++k)
         if (k == at) s[k] = -2.f;
     }
   }
+  if (renorm && lane < top) wts[(int64_t)t * top + lane] = kept_w / (total + 1e-20f) * scale;
 }
 
 extern "C" int ragged_moe_route(const void* x, int64_t ldx, const float* wr, int* idx, float* wts, int64_t rows, int D, int E,
-                                int groups, int keep, int top, float scale, int dtype, hipStream_t st) {
+                                int groups, int keep, int top, float scale, int score_fn, int group_top, int renorm, int dtype,
+                                hipStream_t st) {
+  if (score_fn < 0 || score_fn > 1 || group_top < 1 || group_top > 2 || (renorm && top > 64)) return -1;
   if (rows <= 0 || rows > 0x7fffffff || D <= 0 || D > 12288 || E <= 0 || E > MOE_MAX_E || groups <= 0 || groups > 64 || E % groups) return -1;
   if (keep <= 0 || keep > groups || top <= 0 || top > keep * (E / groups)) return -1;
   RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((moe_route_kernel<T>), dim3((unsigned)rows), dim3(256), D * sizeof(float), st, (const T*)x, ldx, wr, idx,
-                                            wts, D, E, groups, keep, top, scale))
+                                            wts, D, E, groups, keep, top, scale, score_fn, group_top, renorm))
   return RAGGED_LAUNCH_OK();
 }
 
@@ -208,8 +231,10 @@ __device__ __forceinline__ void rows_dot(const T* __restrict__ w, int64_t K, int
 
 constexpr int MOE_RW = 4;           // weight rows per wavefront and pass
 
-// A[(t, j), f] = relu(W_up[idx[t, j]][f, :] . x[t, :])^2.  Grid (rows * top, blocks of 4 * MOE_RW inner channels).
-template <typename T>
+// ACT 0: A[(t, j), f] = relu(W_up[idx[t, j]][f, :] . x[t, :])^2.  ACT 1 (gated experts): W_up holds 2 ff rows per expert, the
+// gate row and the up row of inner channel f next to each other (rows 2 f, 2 f + 1), and A[(t, j), f] = silu(gate) * up.
+// Grid (rows * top, blocks of 4 * MOE_RW weight rows); `ff` counts the weight rows of an expert.
+template <typename T, int ACT>
 __global__ __launch_bounds__(256) void moe_rows_up_kernel(const T* __restrict__ x, int64_t ldx, const int* __restrict__ idx,
                                                           const T* __restrict__ w_up, T* __restrict__ A, int D, int ff, int top,
                                                           int vec) {
@@ -225,9 +250,18 @@ __global__ __launch_bounds__(256) void moe_rows_up_kernel(const T* __restrict__ 
   float acc[MOE_RW];
   rows_dot<T, MOE_RW>(w, D, nrows, xs, vec != 0, lane, acc);
 #pragma unroll
-  for (int r = 0; r < MOE_RW; ++r) {
-    const float v = fmaxf(wave_sum(acc[r]), 0.f);
-    if (lane == 0 && r < nrows) A[(int64_t)pair * ff + f0 + r] = from_f<T>(v * v);
+  for (int r = 0; r < MOE_RW; ++r) acc[r] = wave_sum(acc[r]);
+  if (ACT == 1) {
+#pragma unroll
+    for (int r = 0; r < MOE_RW; r += 2)
+      if (lane == 0 && r + 1 < nrows)
+        A[(int64_t)pair * (ff / 2) + (f0 + r) / 2] = from_f<T>(acc[r] / (1.0f + expf(-acc[r])) * acc[r + 1]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < MOE_RW; ++r) {
+      const float v = fmaxf(acc[r], 0.f);
+      if (lane == 0 && r < nrows) A[(int64_t)pair * ff + f0 + r] = from_f<T>(v * v);
+    }
   }
 }
 
@@ -267,15 +301,22 @@ __global__ __launch_bounds__(256) void moe_rows_down_kernel(const T* __restrict_
       }
 }
 
+// act 0: two-matrix experts with relu^2; act 1: gated experts, w_up [E, 2 ff, D] with (gate, up) rows next to each other
 extern "C" int ragged_moe_rows(const void* x, int64_t ldx, const int* idx, const float* wts, const void* w_up, const void* w_dn,
-                               const void* base, void* A, void* y, int64_t rows, int D, int ff, int top, int dtype,
+                               const void* base, void* A, void* y, int64_t rows, int D, int ff, int top, int act, int dtype,
                                hipStream_t st) {
   if (rows <= 0 || D <= 0 || ff <= 0 || top <= 0 || rows * top > 0x7fffffff || D > 12288 || ff > 12288) return -1;
+  if (act < 0 || act > 1) return -1;
   const int per = 4 * MOE_RW;
+  const int wrows = act == 1 ? 2 * ff : ff;
   RAGGED_DISPATCH(dtype,
     const int vu = D % WVec<T>::N == 0; const int vd = ff % WVec<T>::N == 0;
-    hipLaunchKernelGGL((moe_rows_up_kernel<T>), dim3((unsigned)(rows * top), (ff + per - 1) / per), dim3(256), D * sizeof(float), st,
-                       (const T*)x, ldx, idx, (const T*)w_up, (T*)A, D, ff, top, vu);
+    if (act == 1)
+      hipLaunchKernelGGL((moe_rows_up_kernel<T, 1>), dim3((unsigned)(rows * top), (wrows + per - 1) / per), dim3(256), D * sizeof(float),
+                         st, (const T*)x, ldx, idx, (const T*)w_up, (T*)A, D, wrows, top, vu);
+    else
+      hipLaunchKernelGGL((moe_rows_up_kernel<T, 0>), dim3((unsigned)(rows * top), (ff + per - 1) / per), dim3(256), D * sizeof(float), st,
+                         (const T*)x, ldx, idx, (const T*)w_up, (T*)A, D, ff, top, vu);
     hipLaunchKernelGGL((moe_rows_down_kernel<T>), dim3((unsigned)rows, (D + per - 1) / per), dim3(256), ff * sizeof(float), st,
                        (const T*)A, idx, wts, (const T*)w_dn, (const T*)base, (T*)y, D, ff, top, vd))
   return RAGGED_LAUNCH_OK();
@@ -313,6 +354,8 @@ extern "C" int ragged_moe_combine(const void* ys, const int* place, const float*
 // previous step's matrix instructions run, stored to the other of two LDS buffers, and read back as fragments (both
 // operands are K-contiguous, so a fragment is one 16-byte LDS read); one barrier per step.
 // src_row: the activation row behind every sorted place (null: the place itself).  ACT = 1: relu(.)^2 on the way out.
+// ACT = 2: the N output channels are (gate, up) pairs of N / 2 inner channels, out[row, c] = silu(gate_c) * up_c (a lane's
+// four neighbouring channels are two whole pairs; the output rows are N / 2 long).
 typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
 union MoeFrag {
@@ -431,11 +474,17 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(const bf16* __res
   for (int rb = 0; rb < RB; ++rb) {
     const int row = r0 + 16 * rb + lq;
     if (row >= rend) continue;
-    bf16* orow = out + (int64_t)row * N + n0;
+    bf16* orow = out + (ACT == 2 ? (int64_t)row * (N / 2) + n0 / 2 : (int64_t)row * N + n0);
 #pragma unroll
     for (int nb = 0; nb < MG_NB; ++nb) {
       const int n = 16 * nb + 4 * g4;
       if (n0 + n < N) {                                    // N is a multiple of 16: four channels are in or out together
+        if (ACT == 2) {
+          const float g0 = acc[rb][nb][0], g1 = acc[rb][nb][2];
+          const float a0 = g0 / (1.0f + __expf(-g0)) * acc[rb][nb][1], a1 = g1 / (1.0f + __expf(-g1)) * acc[rb][nb][3];
+          *reinterpret_cast<uint32_t*>(orow + n / 2) = (uint32_t)from_f<bf16>(a0).b | ((uint32_t)from_f<bf16>(a1).b << 16);
+          continue;
+        }
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -470,11 +519,16 @@ extern "C" int ragged_moe_grouped_gemm(const void* X, int64_t ldx, const int* sr
   static bool raised = false;                               // two tiles above 64 KB: the limit is raised once per kernel
   if (!raised) {
     if (hipFuncSetAttribute((const void*)moe_grouped_gemm_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
-        hipFuncSetAttribute((const void*)moe_grouped_gemm_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        hipFuncSetAttribute((const void*)moe_grouped_gemm_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+        hipFuncSetAttribute((const void*)moe_grouped_gemm_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return -3;
     raised = true;
   }
-  if (act == 1)
+  if (act < 0 || act > 2) return -1;
+  if (act == 2)
+    hipLaunchKernelGGL((moe_grouped_gemm_kernel<2>), grid, dim3(256), lds, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
+                       seg, tile_e, tile_r0, ntiles, N, K);
+  else if (act == 1)
     hipLaunchKernelGGL((moe_grouped_gemm_kernel<1>), grid, dim3(256), lds, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
                        seg, tile_e, tile_r0, ntiles, N, K);
   else

@@ -529,3 +529,137 @@ extern "C" int ragged_row_norm(const float* x, const float* w, void* out, int64_
                                             rows, n, eps))
   return RAGGED_LAUNCH_OK();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Embedding rows as the float stream: x[t] = scale * table[ids[t]] (+ table2[ids2[t]]), summed in float.  The second
+// table serves embeddings of token pairs (a row chosen by a hash of the previous and the current token).
+template <typename T>
+__global__ __launch_bounds__(256) void embed_rows_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
+                                                         const int64_t* __restrict__ ids2, const T* __restrict__ table2,
+                                                         float scale, float* __restrict__ x, int D) {
+  const int64_t t = blockIdx.x;
+  const T* r1 = table + ids[t] * D;
+  const T* r2 = table2 ? table2 + ids2[t] * D : nullptr;
+  for (int c = threadIdx.x; c < D; c += 256) {
+    float v = to_f(r1[c]) * scale;
+    if (r2) v += to_f(r2[c]);
+    x[t * D + c] = v;
+  }
+}
+
+extern "C" int ragged_embed_rows(const int64_t* ids, const void* table, const int64_t* ids2, const void* table2, float scale,
+                                 float* x, int64_t rows, int D, int dtype, hipStream_t st) {
+  if (rows <= 0 || rows > 0x7fffffff || D <= 0 || !ids || !table || !x || (table2 && !ids2)) return -1;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((embed_rows_kernel<T>), dim3((unsigned)rows), dim3(256), 0, st, ids, (const T*)table, ids2,
+                                            (const T*)table2, scale, x, D))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Pre-norm form: x <- x + y1 (+ y2) on the float stream, then (w_next given) xa = w_next * rmsnorm(x) for the products
+// that read the stream next.  y2 serves blocks whose mixer and feed-forward read the same normed input and are summed
+// into the stream together.  One workgroup per row; NV as in post_norm_add_kernel.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void add_norm_kernel(float* __restrict__ x, const T* __restrict__ y1, const T* __restrict__ y2,
+                                                       const float* __restrict__ w_next, T* __restrict__ xa, int D, float eps) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * D;
+  if (NV > 0) {
+    float xv[NV > 0 ? NV : 1], wn[NV > 0 ? NV : 1];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      const bool ok = c < D;
+      float v = ok ? x[base + c] : 0.f;
+      float s = (ok && y1) ? to_f(y1[base + c]) : 0.f;
+      if (ok && y2) s += to_f(y2[base + c]);
+      v += s;
+      wn[u] = (ok && xa) ? w_next[c] : 0.f;
+      if (ok && (y1 || y2)) x[base + c] = v;
+      xv[u] = v;
+      ss += v * v;
+    }
+    if (!xa) return;
+    const float r = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      if (c < D) xa[base + c] = from_f<T>(xv[u] * r * wn[u]);
+    }
+    return;
+  }
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += 256) {
+    float s = y1 ? to_f(y1[base + c]) : 0.f;
+    if (y2) s += to_f(y2[base + c]);
+    const float v = x[base + c] + s;
+    if (y1 || y2) x[base + c] = v;
+    ss += v * v;
+  }
+  if (!xa) return;
+  const float r = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
+  for (int c = threadIdx.x; c < D; c += 256) xa[base + c] = from_f<T>(x[base + c] * r * w_next[c]);
+}
+
+extern "C" int ragged_add_norm(float* x, const void* y1, const void* y2, const float* w_next, void* xa, int64_t rows, int D,
+                               float eps, int dtype, hipStream_t st) {
+  if (rows <= 0 || D <= 0 || rows > 0x7fffffff || !x || (xa && !w_next) || (y2 && !y1)) return -1;
+  RAGGED_DISPATCH(dtype,
+    if (D <= 1024) hipLaunchKernelGGL((add_norm_kernel<T, 4>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y1, (const T*)y2,
+                                      w_next, (T*)xa, D, eps);
+    else if (D <= 4096) hipLaunchKernelGGL((add_norm_kernel<T, 16>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y1,
+                                           (const T*)y2, w_next, (T*)xa, D, eps);
+    else hipLaunchKernelGGL((add_norm_kernel<T, 0>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y1, (const T*)y2, w_next,
+                            (T*)xa, D, eps))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Activations of a feed-forward's inner channels.  act_cols: out[r, c] = act(P[r, col0 + c]), c < n, with
+// kind 0: gelu through erf, 0.5 z (1 + erf(z / sqrt 2));  1: gelu through tanh, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)));
+// 2: relu(z)^2.  glu_pairs: the inner channels come as neighbouring (gate, up) pairs, out[r, c] = silu(P[r, 2 c]) * P[r, 2 c + 1].
+template <typename T>
+__global__ __launch_bounds__(256) void act_cols_kernel(const T* __restrict__ P, int64_t ldp, int col0, T* __restrict__ out, int64_t rows,
+                                                       int n, int kind) {
+  const int64_t total = rows * n;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / n;
+    const int c = (int)(i % n);
+    const float z = to_f(P[r * ldp + col0 + c]);
+    float v;
+    if (kind == 0) v = 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    else if (kind == 1) v = 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    else { v = fmaxf(z, 0.f); v *= v; }
+    out[i] = from_f<T>(v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void glu_pairs_kernel(const T* __restrict__ P, int64_t ldp, T* __restrict__ out, int64_t rows, int n) {
+  const int64_t total = rows * n;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / n;
+    const int c = (int)(i % n);
+    const float g = to_f(P[r * ldp + 2 * c]), u = to_f(P[r * ldp + 2 * c + 1]);
+    out[i] = from_f<T>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ragged_act_cols(const void* P, int64_t ldp, int col0, void* out, int64_t rows, int n, int kind, int dtype,
+                               hipStream_t st) {
+  if (rows <= 0 || n <= 0 || col0 < 0 || ldp < col0 + n || kind < 0 || kind > 2) return -1;
+  const int64_t blocks = (rows * n + 255) / 256;
+  const unsigned grid = (unsigned)(blocks < 16384 ? blocks : 16384);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((act_cols_kernel<T>), dim3(grid), dim3(256), 0, st, (const T*)P, ldp, col0, (T*)out, rows, n,
+                                            kind))
+  return RAGGED_LAUNCH_OK();
+}
+
+extern "C" int ragged_glu_pairs(const void* P, int64_t ldp, void* out, int64_t rows, int n, int dtype, hipStream_t st) {
+  if (rows <= 0 || n <= 0 || ldp < 2 * n) return -1;
+  const int64_t blocks = (rows * n + 255) / 256;
+  const unsigned grid = (unsigned)(blocks < 16384 ? blocks : 16384);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((glu_pairs_kernel<T>), dim3(grid), dim3(256), 0, st, (const T*)P, ldp, (T*)out, rows, n))
+  return RAGGED_LAUNCH_OK();
+}

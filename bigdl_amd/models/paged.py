@@ -12,6 +12,10 @@ slots.  A layer declares what it keeps with a spec tuple:
     ("tail", rows, channels)               slot   [slots, rows, channels]    activation type
     ("matrix", heads, rows, cols)          slot   [slots, heads, rows, cols] float32
 
+The keys of the spec dictionary name layer executions (a layer that runs twice keeps two caches).  The pool also
+remembers every sequence's last token (host side), which designs with an embedding of token pairs need for the next
+step's first row.
+
 Nothing is cleared when a page or slot is handed out again: attention never looks past a sequence's own length, and
 the kernels treat a sequence whose past length is 0 as one with zero state.
 """
@@ -62,6 +66,7 @@ class PagedStatePool:
         self.free_slots: List[int] = list(range(self.slots))[::-1]
         self.pages_of: Dict[int, List[int]] = {}
         self.len_of: Dict[int, int] = {}
+        self.last_token: Dict[int, int] = {}      # the sequence's last token so far (-1: none yet), for token-pair embeddings
 
     # ---- sequences
     def admit(self) -> int:
@@ -70,11 +75,13 @@ class PagedStatePool:
         slot = self.free_slots.pop()
         self.pages_of[slot] = []
         self.len_of[slot] = 0
+        self.last_token[slot] = -1
         return slot
 
     def release(self, slot: int):
         self.free_pages.extend(reversed(self.pages_of.pop(slot)))
         del self.len_of[slot]
+        del self.last_token[slot]
         self.free_slots.append(slot)
 
     def reserve(self, slot: int, n_new: int) -> List[int]:
@@ -92,8 +99,10 @@ class PagedStatePool:
         length = self.len_of[slot] if slot is not None else 0
         return (length + n_new + PAGE - 1) // PAGE - have <= len(self.free_pages)
 
-    def commit(self, slot: int, n_new: int):
+    def commit(self, slot: int, n_new: int, last_token=None):
         self.len_of[slot] += n_new
+        if last_token is not None:
+            self.last_token[slot] = int(last_token)
 
     def live_tokens(self) -> int:
         return sum(self.len_of.values())

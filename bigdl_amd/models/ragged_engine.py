@@ -10,7 +10,10 @@ into arbitrary portions next to single decoded tokens run here instead:
 * keys / values live in 64-token pages of a ``PagedStatePool``, per-sequence state in its slots;
 * the mixers are described by small dataclasses whose fields are the design's constants, so a new design is a new list
   of them (``models/lipizen.py`` and ``models/merusun.py`` build one from a ``config.json``);
-* two residual forms: the post-sum norm x <- norm(alpha x + f(x)), and the sandwich x <- x + norm_b(f(norm_a(x)));
+* three residual forms: the post-sum norm x <- norm(alpha x + f(x)), the sandwich x <- x + norm_b(f(norm_a(x))), and the
+  parallel pre-norm block u = norm(x), x <- x + mixer(u) + ff(u);
+* a run of layers may be executed several times with the same weights (every execution has its own cache), with the
+  embedding output mixed back into the stream in front of a pass; the embedding may add a row of a token-pair table;
 * matrix products are the library's (bf16 inputs with 32-bit accumulation, or plain float32), everything between them
   is ``ops/ragged.py``.
 """
@@ -53,6 +56,12 @@ class WindowAttention:
     kv_from: Optional[int] = None  # read this layer's cache instead of projecting keys / values
     bias: bool = False             # the q / k / v projections have biases
     sink: Optional[float] = None   # score of a key without a value that every query sees: exp(sink) joins the normaliser
+    chunk: int = 0                 # > 0: keys are visible only inside the query's block of this many positions (from position 0)
+    softcap: float = 0.0           # > 0: score <- softcap * tanh(score / softcap), after the scale
+    rot_neighbours: bool = False   # rotated pairs are (2 i, 2 i + 1) instead of (i, i + rot_dims / 2)
+    rot_freqs: Optional[tuple] = None  # the pairs' frequencies, if they are not base^(-2 i / rot_dims) / rot_factor
+    rot_amp: float = 1.0           # cosine and sine are multiplied by this
+    gate_channels: bool = False    # with ``gate``: one sigmoid gate per output channel instead of one per head
 
 
 @dataclass
@@ -104,9 +113,11 @@ class ClampedGlu:
 
 @dataclass
 class RoutedExperts:
-    """Mixture of two-matrix experts y = W_down act(W_up h), act = relu squared.  Scores are a softmax over all experts'
-    router logits (32-bit); experts come in ``groups`` equal runs of neighbours, a group scores as its best expert, and
-    the ``top`` best experts inside the ``keep`` best groups are used, weighted by score * ``scale`` (not renormalised).
+    """Mixture of small experts.  ``act`` "relu2": y = W_down relu(W_up h)^2; "swiglu": y = W_down (silu(W_gate h) * W_up h)
+    (``LayerTensors.w_up`` then holds the gate and up rows of an inner channel next to each other).  Scores are a softmax
+    over all experts' router logits or a sigmoid per expert (32-bit); experts come in ``groups`` equal runs of neighbours,
+    a group scores as the sum of its ``group_top`` best experts, and the ``top`` best experts inside the ``keep`` best
+    groups are used, weighted by score * ``scale``, the scores first divided by their sum (+ 1e-20) with ``renorm``.
     ``shared_ff`` > 0: one more expert of that inner size that every token uses with weight 1."""
     experts: int
     top: int
@@ -115,6 +126,37 @@ class RoutedExperts:
     keep: int = 1
     scale: float = 1.0
     shared_ff: int = 0
+    score: str = "softmax"         # or "sigmoid"
+    group_top: int = 1
+    renorm: bool = False
+    act: str = "relu2"             # or "swiglu"
+
+
+@dataclass
+class DenseMlp:
+    """y = W_down act(W_up h + b_up) + b_down, act "gelu_erf" (0.5 z (1 + erf(z / sqrt 2))), "gelu_tanh" or "relu2".  In the
+    parallel block its up projection is stacked behind the mixer's input projections (one product reads the normed
+    stream once)."""
+    ff: int
+    act: str = "gelu_erf"
+    bias: bool = True
+
+
+@dataclass
+class PairEmbedding:
+    """A second embedding table indexed by a hash of (previous token, token): row (prev * mul_prev + cur * mul_cur) mod
+    buckets; a sequence's first token, which has no previous one, takes row ``buckets`` (the table's last)."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+
+    def rows(self, prev: int, tokens: Sequence[int]) -> List[int]:
+        """``prev``: the sequence's last token so far, -1 for a new sequence"""
+        out = []
+        for t in tokens:
+            out.append(self.buckets if prev < 0 else (prev * self.mul_prev + int(t) * self.mul_cur) % self.buckets)
+            prev = int(t)
+        return out
 
 
 @dataclass
@@ -129,7 +171,15 @@ class RaggedConfig:
     logit_softcap: float = 0.0
     name: str = "ragged"
     embed_scale: float = 1.0
-    block: str = "post_sum"        # "post_sum": x <- norm(alpha x + f(x)); "sandwich": x <- x + norm_b(f(norm_a(x)))
+    block: str = "post_sum"        # "post_sum": x <- norm(alpha x + f(x)); "sandwich": x <- x + norm_b(f(norm_a(x)));
+                                   # "parallel": u = norm(x), x <- x + mixer(u) + ff(u)
+    runs: Optional[list] = None    # layer index of every layer execution, in order (None: every layer once); an execution
+                                   # has its own cache / state, whatever weights it shares
+    mix_in: tuple = ()             # executions in front of which x <- W_mix [x ; embedding output]
+    pair_embed: Optional[PairEmbedding] = None
+
+    def layer_runs(self) -> list:
+        return list(range(len(self.mixers))) if self.runs is None else list(self.runs)
 
 
 @dataclass
@@ -158,6 +208,7 @@ class LayerTensors:
     w_dn: Optional[torch.Tensor] = None      # [experts, width, ff]
     w_sup: Optional[torch.Tensor] = None     # shared expert
     w_sdn: Optional[torch.Tensor] = None
+    b_down: Optional[torch.Tensor] = None    # dense feed-forward: bias of the down projection (the up bias is part of b_in)
 
 
 def rotary_inv_freq(dims: int, base: float, factor: float) -> torch.Tensor:
@@ -166,23 +217,58 @@ def rotary_inv_freq(dims: int, base: float, factor: float) -> torch.Tensor:
     return (float(base) ** (-2.0 * i / dims)) / float(factor)
 
 
+def yarn_inv_freq(dims: int, base: float, factor: float, original: float, fast: float, slow: float):
+    """Frequencies of a rotation stretched for contexts longer than the ``original`` one, pair by pair: with
+    index(t) = dims ln(original / (2 pi t)) / (2 ln base) the pair whose wavelength turns t times in the original context,
+    lo = max(floor(index(fast)), 0), hi = min(ceil(index(slow)), dims - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
+    f_i' = r_i f_i / factor + (1 - r_i) f_i: fast pairs keep their frequency, slow ones are divided by ``factor``.
+    Returns (float32 frequencies, amplitude 0.1 ln(factor) + 1 that multiplies cosine and sine)."""
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+
+    def index(turns):
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+    lo, hi = max(math.floor(index(fast)), 0), min(math.ceil(index(slow)), dims - 1)
+    out = []
+    for i, fi in enumerate(f):
+        r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        out.append(fi / factor * r + fi * (1.0 - r))
+    return torch.tensor(out, dtype=torch.float64).to(torch.float32), 0.1 * math.log(factor) + 1.0
+
+
 class RaggedDecoder:
     ragged = True                  # serving/continuous.py steps such an engine with mixed batches
 
     def __init__(self, cfg: RaggedConfig, embed: torch.Tensor, layers: List[LayerTensors], final_norm: torch.Tensor,
-                 head: torch.Tensor, act_dtype=torch.bfloat16, device="cuda"):
+                 head: torch.Tensor, act_dtype=torch.bfloat16, device="cuda", pair_table: Optional[torch.Tensor] = None,
+                 w_mix: Optional[torch.Tensor] = None):
+        """``pair_table`` [buckets + 1, width]: the token-pair embedding of ``cfg.pair_embed``; ``w_mix`` [width, 2 width]:
+        the projection of [stream ; embedding output] in front of the executions named in ``cfg.mix_in``."""
         self.cfg, self.embed, self.layers, self.final_norm, self.head = cfg, embed, layers, final_norm, head
+        self.pair_table, self.w_mix = pair_table, w_mix
         self.act = act_dtype
         self.device = torch.device(device)
         self.ops = R.ops_for(self.device)
         self.pool: Optional[PagedStatePool] = None
-        for li, m in enumerate(cfg.mixers):
+        self.runs = cfg.layer_runs()
+        if any(not 0 <= li < len(layers) for li in self.runs) or any(not 0 <= ri < len(self.runs) for ri in cfg.mix_in):
+            raise ValueError("layer executions outside the layer list")
+        if cfg.mix_in and (w_mix is None or tuple(w_mix.shape) != (cfg.width, 2 * cfg.width) or cfg.block != "parallel"):
+            raise ValueError("mixing the embedding output back in needs a [width, 2 width] projection and the parallel block")
+        if cfg.pair_embed is not None and (pair_table is None or tuple(pair_table.shape) != (cfg.pair_embed.buckets + 1, cfg.width)):
+            raise ValueError("the token-pair table must have buckets + 1 rows of the stream's width")
+        self._kv_run = {}                  # execution -> the execution whose cache it reads (itself unless kv_from is set)
+        latest = {}
+        for ri, li in enumerate(self.runs):
+            m = cfg.mixers[li]
+            self._kv_run[ri] = ri
             if isinstance(m, WindowAttention) and m.kv_from is not None:
-                o = cfg.mixers[m.kv_from] if 0 <= m.kv_from < li else None
+                o = cfg.mixers[m.kv_from] if 0 <= m.kv_from < len(cfg.mixers) and m.kv_from in latest else None
                 if not isinstance(o, WindowAttention) or o.kv_from is not None or \
                         (o.kv_heads, o.dim, o.vdim, o.maps) != (m.kv_heads, m.dim, m.vdim, m.maps):
                     raise ValueError(f"layer {li}: kv_from must name an earlier attention layer with keys of its own and "
                                      "the same head layout")
+                self._kv_run[ri] = latest[m.kv_from]
+            latest[li] = ri
         self.first_cost = self.rest_cost_mean = self.peak_memory = 0.0
         # BIGDL_RAGGED_GRAPH=1: steps that carry one token per sequence are recorded once per (sequences, page-table
         # width) and replayed as one hipGraph.  Off by default: every step is issued kernel by kernel.  With recording
@@ -193,8 +279,10 @@ class RaggedDecoder:
 
     # ------------------------------------------------------------------ state
     def state_specs(self):
+        """what every layer execution keeps, by execution index"""
         specs = {}
-        for li, m in enumerate(self.cfg.mixers):
+        for ri, li in enumerate(self.runs):
+            m = self.cfg.mixers[li]
             s = []
             if isinstance(m, WindowAttention):
                 if m.kv_from is None:
@@ -208,7 +296,7 @@ class RaggedDecoder:
             elif isinstance(m, Mlstm):
                 s.append(("matrix", m.heads, m.dim, m.vdim + 1))  # S and, as its last column, the normaliser n
                 s.append(("vector", m.heads))                   # the running maximum of every head
-            specs[li] = s
+            specs[ri] = s
         return specs
 
     @staticmethod
@@ -227,27 +315,30 @@ class RaggedDecoder:
 
     # ------------------------------------------------------------------ layers
     def _attention(self, li, m: WindowAttention, lt: LayerTensors, P, meta):
+        """``li`` (here and in the other mixers): the execution's index, which names its cache / state in the pool"""
         ops, pool, eps = self.ops, self.pool, self.cfg.norm_eps
+        turn = dict(interleaved=m.rot_neighbours, rot_amp=m.rot_amp)
         cq = m.heads * m.maps * m.dim
         ck = m.kv_heads * m.maps * m.dim
         conv = dict(cw=lt.conv_w, taps=m.conv_taps, C=self._conv_channels(m), state=pool.tail.get(li)) if m.conv_taps else \
             dict(cw=None, taps=0, C=0, state=None)
         q = torch.empty(meta.T, cq, dtype=torch.float32, device=self.device)
         ops.conv_head(P, 0, meta, ch0=0, ngroups=m.heads * m.maps, gsize=m.dim, normw=lt.q_norm, eps=eps, rot=m.rot_dims,
-                      inv_freq=lt.inv_freq, out_dense=q, **conv)
+                      inv_freq=lt.inv_freq, out_dense=q, **conv, **turn)
         col = cq
         if m.kv_from is None:
             ops.conv_head(P, cq, meta, ch0=cq, ngroups=m.kv_heads * m.maps, gsize=m.dim, normw=lt.k_norm, eps=eps,
-                          rot=m.rot_dims, inv_freq=lt.inv_freq, pages=pool.k[li], **conv)
+                          rot=m.rot_dims, inv_freq=lt.inv_freq, pages=pool.k[li], **conv, **turn)
             ops.conv_head(P, cq + ck, meta, ch0=cq + ck, ngroups=m.kv_heads, gsize=m.vdim, normw=None, eps=eps, rot=0,
                           inv_freq=None, pages=pool.v[li], **conv)
             col = cq + ck + m.kv_heads * m.vdim
         if m.conv_taps > 1:
             ops.conv_state(P, 0, pool.tail[li], m.conv_taps, conv["C"], meta)
-        src = li if m.kv_from is None else m.kv_from
+        src = self._kv_run[li]
         return ops.paged_attn(q, pool.k[src], pool.v[src], meta, maps=m.maps, H=m.heads, G=m.kv_heads, d=m.dim, vd=m.vdim,
                               window=m.window, keep_first=m.keep_first, scale=m.scale, lam=m.lam, out_scale=m.out_scale,
-                              out_norm=m.out_norm, eps=eps, gate=P if m.gate else None, gate0=col, sink=m.sink)
+                              out_norm=m.out_norm, eps=eps, gate=P if m.gate else None, gate0=col, sink=m.sink,
+                              chunk=m.chunk, softcap=m.softcap, gate_wide=m.gate and m.gate_channels)
 
     def _latent(self, li, m: LatentAttention, lt: LayerTensors, P, meta):
         """Scores of head h are q_h . [W_uk,h c | rotated part] = [W_uk,h^T q_h | rotated query part] . [c | rotated part]:
@@ -286,13 +377,15 @@ class RaggedDecoder:
 
     def _experts(self, f: RoutedExperts, lt: LayerTensors, xa, meta):
         ops = self.ops
-        idx, wts = ops.moe_route(xa, lt.w_router, f.groups, f.keep, f.top, f.scale)
+        gated = f.act == "swiglu"
+        idx, wts = ops.moe_route(xa, lt.w_router, f.groups, f.keep, f.top, f.scale, f.score, f.group_top, f.renorm)
         base = None
         if f.shared_ff:
-            base = F.linear(ops.relu2(F.linear(xa, lt.w_sup)), lt.w_sdn)
+            a = F.linear(xa, lt.w_sup)
+            base = F.linear(ops.glu_pairs(a) if gated else ops.relu2(a), lt.w_sdn)
         if meta.T * f.top < self.moe_dense_rows * f.experts:
-            return ops.moe_rows(xa, idx, wts, lt.w_up, lt.w_dn, base)
-        y = ops.moe_sorted(xa, idx, wts, lt.w_up, lt.w_dn, base)                # bfloat16: one grouped product per projection
+            return ops.moe_rows(xa, idx, wts, lt.w_up, lt.w_dn, base, gated)
+        y = ops.moe_sorted(xa, idx, wts, lt.w_up, lt.w_dn, base, gated)         # bfloat16: one grouped product per projection
         if y is not None:
             return y
         # rows sorted by expert: one gather, two library products per expert on its run of rows, one weighted sum per row
@@ -301,13 +394,13 @@ class RaggedDecoder:
         counts = torch.bincount(order.values, minlength=f.experts).tolist()     # (the host learns the runs' lengths)
         pair = order.indices                                                    # pair t * top + j at every sorted place
         xs = xa[pair // top]
-        A = torch.empty(T * top, f.ff, dtype=self.act, device=self.device)
+        A = torch.empty(T * top, lt.w_up.shape[1], dtype=self.act, device=self.device)
         at = 0
         for e, c in enumerate(counts):
             if c:
                 torch.mm(xs[at:at + c], lt.w_up[e].t(), out=A[at:at + c])
                 at += c
-        A = ops.relu2(A)
+        A = ops.glu_pairs(A) if gated else ops.relu2(A)
         ys = torch.empty(T * top, self.cfg.width, dtype=self.act, device=self.device)
         at = 0
         for e, c in enumerate(counts):
@@ -332,12 +425,15 @@ class RaggedDecoder:
         these tokens.  ``want[i]``: indices into entry i's tokens whose logits are returned (default: the last one).
         Returns float32 logits [wanted rows, vocab] in the order of entries and indices."""
         pool = self.pool
-        seqs, ids = [], []
+        pairs = self.cfg.pair_embed
+        seqs, ids, prs = [], [], []
         for slot, toks in entries:
             if len(toks) == 0:
                 raise ValueError("an entry without tokens")
             seqs.append((slot, pool.len_of[slot], len(toks), list(pool.reserve(slot, len(toks)))))
             ids += list(toks)
+            if pairs is not None:                    # the previous token is part of the sequence's state
+                prs += pairs.rows(pool.last_token[slot], toks)
         rows, at = [], 0
         for b, (_, _, n, _) in enumerate(seqs):
             idx = [n - 1] if want is None else want[b]
@@ -345,15 +441,15 @@ class RaggedDecoder:
                 raise ValueError("a wanted index outside its entry")
             rows += [at + i for i in idx]
             at += n
-        idt = torch.tensor(ids, dtype=torch.int64)
+        idt = torch.tensor(ids if pairs is None else [ids, prs], dtype=torch.int64)      # [T], or [2, T] with pair rows
         if self.use_graph and collect is None and len(ids) == len(seqs) and rows == list(range(len(seqs))):
             logits = self._decode_step(seqs, idt)
         else:
             if self.device.type == "cuda":
                 idt = idt.pin_memory().to(self.device, non_blocking=True)
             logits = self._forward(R.BatchMeta(seqs, self.device), idt, rows, collect)
-        for slot, _, n, _ in seqs:
-            pool.commit(slot, n)
+        for (slot, _, n, _), (_, toks) in zip(seqs, entries):
+            pool.commit(slot, n, last_token=int(toks[-1]))
         return logits
 
     def _decode_step(self, seqs, idt):
@@ -371,8 +467,8 @@ class RaggedDecoder:
                                  list(range(B)), None)
         if not ent:
             ent["meta"] = R.BatchMeta(seqs, self.device, max_pages=width, static=True)
-            ent["host_ids"] = torch.empty(B, dtype=torch.int64, pin_memory=True)
-            ent["ids"] = torch.zeros(B, dtype=torch.int64, device=self.device)
+            ent["host_ids"] = torch.empty(idt.shape, dtype=torch.int64, pin_memory=True)
+            ent["ids"] = torch.zeros(idt.shape, dtype=torch.int64, device=self.device)
             self.ops.before_recording(ent["meta"])       # whatever the operations would otherwise build on first use
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -400,15 +496,19 @@ class RaggedDecoder:
 
     def _forward(self, meta, idt, rows, collect):
         cfg, ops = self.cfg, self.ops
-        x = F.embedding(idt, self.embed).float()
-        if cfg.embed_scale != 1.0:
-            x = x * cfg.embed_scale
+        if cfg.pair_embed is not None:
+            x = ops.embed_rows(idt[0], self.embed, idt[1], self.pair_table, cfg.embed_scale)
+        else:
+            x = ops.embed_rows(idt, self.embed, scale=cfg.embed_scale)
         if cfg.block == "sandwich":
             self._sandwich_layers(x, meta, collect)
+        elif cfg.block == "parallel":
+            x = self._parallel_layers(x, meta, collect)
         else:
             xa = x.to(self.act)
-            for li, (m, mlp, lt) in enumerate(zip(cfg.mixers, cfg.mlps, self.layers)):
-                a = self._mixer(li, m, lt, F.linear(xa, lt.w_in, lt.b_in), meta)
+            for ri, li in enumerate(self.runs):
+                m, mlp, lt = cfg.mixers[li], cfg.mlps[li], self.layers[li]
+                a = self._mixer(ri, m, lt, F.linear(xa, lt.w_in, lt.b_in), meta)
                 xa = ops.sum_group_norm(x, F.linear(a, lt.w_out), lt.norm1, cfg.norm_groups, cfg.residual_alpha, cfg.norm_eps,
                                         self.act)
                 if mlp is not None:
@@ -434,11 +534,12 @@ class RaggedDecoder:
         """x <- x + norm_b(f(norm_a(x))) for the mixer and the feed-forward of every layer; x float32, in place.  The norm
         behind a sublayer, the residual sum and the norm in front of the next sublayer are one kernel."""
         cfg, ops, eps = self.cfg, self.ops, self.cfg.norm_eps
-        n = len(self.layers)
-        xa = ops.row_norm(x, self.layers[0].norm1, eps, self.act) if n else None
-        for li, (m, mlp, lt) in enumerate(zip(cfg.mixers, cfg.mlps, self.layers)):
-            nxt = self.layers[li + 1].norm1 if li + 1 < n else None
-            a = self._mixer(li, m, lt, F.linear(xa, lt.w_in, lt.b_in), meta)
+        n = len(self.runs)
+        xa = ops.row_norm(x, self.layers[self.runs[0]].norm1, eps, self.act) if n else None
+        for ri, li in enumerate(self.runs):
+            m, mlp, lt = cfg.mixers[li], cfg.mlps[li], self.layers[li]
+            nxt = self.layers[self.runs[ri + 1]].norm1 if ri + 1 < n else None
+            a = self._mixer(ri, m, lt, F.linear(xa, lt.w_in, lt.b_in), meta)
             xa = ops.post_norm_add(x, F.linear(a, lt.w_out), lt.norm1b, nxt if mlp is None else lt.norm2, eps, self.act)
             if isinstance(mlp, RoutedExperts):
                 xa = ops.post_norm_add(x, self._experts(mlp, lt, xa, meta), lt.norm2b, nxt, eps, self.act)
@@ -446,6 +547,43 @@ class RaggedDecoder:
                 raise ValueError("the sandwich form has no such feed-forward yet")
             if collect is not None:
                 collect.append(x.clone())
+
+    def _parallel_layers(self, x, meta, collect):
+        """u = norm(x), x <- x + mixer(u) + ff(u): both sublayers read one normed copy of the stream, their outputs join it
+        in one kernel that also norms the stream for the next execution.  In front of the executions of ``cfg.mix_in``
+        the stream becomes W_mix [x ; e], e the embedding output (bfloat16 operands, 32-bit result)."""
+        cfg, ops, eps = self.cfg, self.ops, self.cfg.norm_eps
+        mix_in = set(cfg.mix_in)
+        e_act = x.to(self.act, copy=True) if mix_in else None      # (the stream itself is updated in place below)
+        n, xa = len(self.runs), None
+        for ri, li in enumerate(self.runs):
+            m, mlp, lt = cfg.mixers[li], cfg.mlps[li], self.layers[li]
+            if ri in mix_in:
+                x = self._linear_f32(torch.cat([x.to(self.act), e_act], 1), self.w_mix)
+                xa = None
+            if xa is None:
+                xa = ops.add_norm(x, None, None, lt.norm1, eps, self.act)
+            P = F.linear(xa, lt.w_in, lt.b_in)       # [mixer's projections | up projection of a dense feed-forward]
+            y1 = F.linear(self._mixer(ri, m, lt, P, meta), lt.w_out)
+            if isinstance(mlp, DenseMlp):
+                y2 = F.linear(ops.act_cols(P, P.shape[1] - mlp.ff, mlp.ff, mlp.act), lt.w_down, lt.b_down)
+            elif isinstance(mlp, RoutedExperts):
+                y2 = self._experts(mlp, lt, xa, meta)
+            elif mlp is None:
+                y2 = None
+            else:
+                raise ValueError("the parallel block has no such feed-forward")
+            nxt = self.layers[self.runs[ri + 1]].norm1 if ri + 1 < n and ri + 1 not in mix_in else None
+            xa = ops.add_norm(x, y1, y2, nxt, eps, self.act)
+            if collect is not None:
+                collect.append(x.clone())
+        return x
+
+    def _linear_f32(self, a, w):
+        """a w^T with the operands in the activation type and a float32 result (no rounding of the 32-bit accumulator)"""
+        if a.dtype == torch.float32 or a.device.type != "cuda":
+            return F.linear(a.float(), w.float())
+        return torch.mm(a, w.t(), out_dtype=torch.float32)
 
     # ------------------------------------------------------------------ generation
     @torch.no_grad()
@@ -472,7 +610,7 @@ class RaggedDecoder:
         return out
 
     def weight_bytes(self):
-        ts = [self.embed, self.head, self.final_norm]
+        ts = [self.embed, self.head, self.final_norm] + [t for t in (self.pair_table, self.w_mix) if t is not None]
         for lt in self.layers:
             ts += [t for t in vars(lt).values() if isinstance(t, torch.Tensor)]
         return sum(t.numel() * t.element_size() for t in ts)

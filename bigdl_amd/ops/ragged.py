@@ -74,7 +74,8 @@ class _AttnArgs(ctypes.Structure):
                 ("keep_first", ctypes.c_int), ("scale", ctypes.c_float), ("lam", ctypes.c_float),
                 ("out_scale", ctypes.c_float), ("out_norm", ctypes.c_int), ("eps", ctypes.c_float),
                 ("rows", ctypes.c_void_p), ("n_rows", ctypes.c_int), ("tiles", ctypes.c_void_p), ("n_tiles", ctypes.c_int),
-                ("ldv", ctypes.c_int64), ("sink", ctypes.c_int), ("sink_score", ctypes.c_float)]
+                ("ldv", ctypes.c_int64), ("sink", ctypes.c_int), ("sink_score", ctypes.c_float), ("chunk", ctypes.c_int),
+                ("softcap", ctypes.c_float), ("gate_wide", ctypes.c_int)]
 
 
 def lib():
@@ -94,13 +95,17 @@ def lib():
         L.ragged_mlstm_gates.argtypes = [vp, i64, ci, vp, cf, cf, vp, vp, vp, vp, ci, _Batch, ci, vp]
         L.ragged_mlstm_expand.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
         L.ragged_head_norm_gate.argtypes = [vp, vp, vp, i64, ci, vp, i64, ci, ci, cf, ci, vp, cf, ci, vp]
-        L.ragged_moe_route.argtypes = [vp, i64, vp, vp, vp, i64, ci, ci, ci, ci, ci, cf, ci, vp]
+        L.ragged_moe_route.argtypes = [vp, i64, vp, vp, vp, i64, ci, ci, ci, ci, ci, cf, ci, ci, ci, ci, vp]
+        L.ragged_embed_rows.argtypes = [vp, vp, vp, vp, cf, vp, i64, ci, ci, vp]
+        L.ragged_add_norm.argtypes = [vp, vp, vp, vp, vp, i64, ci, cf, ci, vp]
+        L.ragged_act_cols.argtypes = [vp, i64, ci, vp, i64, ci, ci, ci, vp]
+        L.ragged_glu_pairs.argtypes = [vp, i64, vp, i64, ci, ci, vp]
         L.ragged_relu2.argtypes = [vp, vp, i64, ci, vp]
         L.ragged_moe_combine.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
         L.ragged_moe_grouped_ok.argtypes = [ci, ci, ci]
         L.ragged_moe_tile_map.argtypes = [vp, ci, vp, vp, vp, ci, vp]
         L.ragged_moe_grouped_gemm.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
-        L.ragged_moe_rows.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, ci, vp]
+        L.ragged_moe_rows.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, ci, ci, vp]
         L.ragged_hgrn2_chunk_decay.argtypes = [vp, vp, vp, ci, ci, vp]
         L.ragged_hgrn2_chunk_combine.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
         L.ragged_row_norm.argtypes = [vp, vp, vp, i64, ci, cf, ci, vp]
@@ -190,13 +195,14 @@ class BatchMeta:
             self._chunks[length] = (nc, buf[o[0]:o[1]], buf[o[1]:o[2]], buf[o[2]:o[3]], buf[o[3]:o[4]], buf[o[4]:], last)
         return self._chunks[length]
 
-    def cossin(self, inv_freq: torch.Tensor) -> torch.Tensor:
-        """[T, rot / 2, 2] float32: cos and sin of position * frequency for every row, made once per step and set of
-        frequencies with the library's full-precision functions (the angle itself is the float32 product)."""
-        key = inv_freq.data_ptr()
+    def cossin(self, inv_freq: torch.Tensor, amp: float = 1.0) -> torch.Tensor:
+        """[T, rot / 2, 2] float32: ``amp`` times cos and sin of position * frequency for every row, made once per step
+        and set of frequencies with the library's full-precision functions (the angle itself is the float32 product)."""
+        key = (inv_freq.data_ptr(), float(amp))
         if key not in self._rot:
             ang = self.tok_pos.to(inv_freq.device).float()[:, None] * inv_freq[None]
-            self._rot[key] = torch.stack([ang.cos(), ang.sin()], -1).contiguous()
+            tab = torch.stack([ang.cos(), ang.sin()], -1)
+            self._rot[key] = (tab * float(amp) if amp != 1.0 else tab).contiguous()
         return self._rot[key]
 
     def attn_split(self, min_rows: int):
@@ -280,7 +286,7 @@ class HipOps:
         return xa
 
     def conv_head(self, P, col0, meta, *, cw, taps, C, ch0, state, ngroups, gsize, normw, eps, rot, inv_freq,
-                  out_dense=None, pages=None, norm_n=None, rot0=0, interleaved=False):
+                  out_dense=None, pages=None, norm_n=None, rot0=0, interleaved=False, rot_amp=1.0):
         _act(P, state, pages)
         _f32(cw, normw, inv_freq, out_dense)
         if P.dim() != 2 or P.shape[0] != meta.T or col0 < 0 or col0 + ngroups * gsize > P.shape[1]:
@@ -303,7 +309,7 @@ class HipOps:
         if rot:
             if inv_freq.numel() != rot // 2 or rot % 2 or rot0 < 0 or rot0 + rot > gsize:
                 raise ValueError("one frequency per rotated pair, pairs inside the group")
-            a.rot, a.cossin, a.rot0, a.interleaved = rot, meta.cossin(inv_freq).data_ptr(), rot0, int(bool(interleaved))
+            a.rot, a.cossin, a.rot0, a.interleaved = rot, meta.cossin(inv_freq, rot_amp).data_ptr(), rot0, int(bool(interleaved))
         if out_dense is not None:
             if out_dense.shape != (meta.T, ngroups * gsize):
                 raise ValueError("dense output shape")
@@ -412,8 +418,10 @@ class HipOps:
         return out
 
     def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
-                   eps, gate=None, gate0=0, sink=None):
-        """``vpages`` may be ``kpages`` itself: the values are then the leading ``vd`` channels of the key rows."""
+                   eps, gate=None, gate0=0, sink=None, chunk=0, softcap=0.0, gate_wide=False):
+        """``vpages`` may be ``kpages`` itself: the values are then the leading ``vd`` channels of the key rows.
+        ``chunk`` > 0: a key is visible only inside the query's block of that many positions; ``softcap`` > 0: scores go
+        through softcap * tanh(. / softcap); ``gate_wide``: one gate column per output channel instead of one per head."""
         _f32(q)
         _act(kpages, vpages, gate)
         _page_check(meta, kpages)
@@ -427,9 +435,12 @@ class HipOps:
         a = _AttnArgs()
         a.q, a.kpages, a.vpages, a.out = q.data_ptr(), kpages.data_ptr(), vpages.data_ptr(), out.data_ptr()
         if gate is not None:
-            if gate.shape[0] != meta.T or gate0 + H > gate.shape[1] or gate.dtype != kpages.dtype:
+            if gate.shape[0] != meta.T or gate0 + (H * vd if gate_wide else H) > gate.shape[1] or gate.dtype != kpages.dtype:
                 raise ValueError("gate columns outside the projection matrix")
-            a.gate, a.ldg, a.gate0 = gate.data_ptr(), gate.stride(0), gate0
+            a.gate, a.ldg, a.gate0, a.gate_wide = gate.data_ptr(), gate.stride(0), gate0, int(bool(gate_wide))
+        if chunk < 0 or softcap < 0:
+            raise ValueError("block size and score cap cannot be negative")
+        a.chunk, a.softcap = int(chunk), float(softcap)
         a.H, a.G, a.d, a.vd, a.window, a.keep_first = H, G, d, vd, window, keep_first
         a.scale, a.lam, a.out_scale, a.out_norm, a.eps = scale, lam, out_scale, int(out_norm), eps
         a.ldv = vpages.shape[3]
@@ -437,7 +448,7 @@ class HipOps:
             a.sink, a.sink_score = 1, float(sink)
         if kpages.dtype == torch.bfloat16 and self.mfma and maps == 1 and not lib().ragged_paged_attn_mfma_ok(d, vd) \
                 and lib().ragged_paged_attn_mfma_wide_ok(d, vd) and a.ldv % 8 == 0 and not keep_first and not out_norm \
-                and gate is None:
+                and gate is None and not chunk and not softcap:
             # rows too wide for the row-wise kernel's lanes: long portions as tiles of 64 rows of one head, single tokens
             # and short portions with 16 heads of a row side by side, both on the matrix cores
             tiles, n_tiles, rows, n_rows = meta.attn_split(self.mfma_min_rows)
@@ -448,7 +459,8 @@ class HipOps:
                 a.rows, a.n_rows = rows.data_ptr(), n_rows
                 _ok(lib().ragged_paged_attn_mfma_heads(a, meta.c(), _stream()), "paged_attn_mfma_heads")
             return out
-        if kpages.dtype == torch.bfloat16 and self.mfma and lib().ragged_paged_attn_mfma_ok(d, vd) and a.ldv % 8 == 0:
+        if kpages.dtype == torch.bfloat16 and self.mfma and lib().ragged_paged_attn_mfma_ok(d, vd) and a.ldv % 8 == 0 \
+                and not (gate_wide and (a.ldg % 4 or gate0 % 4)):
             # long portions on the matrix cores, single tokens and short portions row by row
             tiles, n_tiles, rows, n_rows = meta.attn_split(self.mfma_min_rows)
             if n_tiles:
@@ -526,7 +538,9 @@ class HipOps:
                                       gf.data_ptr(), T, H, d, _DT[P.dtype], _stream()), "mlstm_expand")
         return qf, ff, gf
 
-    def moe_route(self, xa, w_router, groups, keep, top, scale):
+    def moe_route(self, xa, w_router, groups, keep, top, scale, score="softmax", group_top=1, renorm=False):
+        """``score``: "softmax" over all experts or "sigmoid" per expert; a group is worth the sum of its ``group_top``
+        best scores; ``renorm``: the chosen scores are divided by their sum (+ 1e-20) before ``scale``."""
         _act(xa)
         _f32(w_router)
         T, D = xa.shape
@@ -536,19 +550,21 @@ class HipOps:
         idx = torch.empty(T, top, dtype=torch.int32, device=xa.device)
         wts = torch.empty(T, top, dtype=torch.float32, device=xa.device)
         _ok(lib().ragged_moe_route(xa.data_ptr(), xa.stride(0), w_router.data_ptr(), idx.data_ptr(), wts.data_ptr(), T, D, E, groups,
-                                   keep, top, scale, _DT[xa.dtype], _stream()), "moe_route")
+                                   keep, top, scale, {"softmax": 0, "sigmoid": 1}[score], int(group_top), int(bool(renorm)),
+                                   _DT[xa.dtype], _stream()), "moe_route")
         return idx, wts
 
-    def moe_sorted(self, xa, idx, wts, w_up, w_dn, base):
+    def moe_sorted(self, xa, idx, wts, w_up, w_dn, base, gated=False):
         """The experts of long bfloat16 portions without a word to the host: (row, choice) pairs sorted by expert, every
-        expert's run cut into 64-row tiles on the device, one grouped matrix-core product for all up projections (relu^2
-        on the way out) and one for all down projections, then every row's weighted sum.  None when the sizes are not
-        served (the caller then runs the experts one by one)."""
+        expert's run cut into 64-row tiles on the device, one grouped matrix-core product for all up projections (relu^2,
+        or with ``gated`` silu(gate) * up over neighbouring weight rows, on the way out) and one for all down projections,
+        then every row's weighted sum.  None when the sizes are not served (the caller then runs the experts one by one)."""
         T, D = xa.shape
-        E, ff, top = w_up.shape[0], w_up.shape[1], idx.shape[1]
+        E, wrows, top = w_up.shape[0], w_up.shape[1], idx.shape[1]
+        ff = wrows // 2 if gated else wrows
         L = lib()
-        if xa.dtype != torch.bfloat16 or not (L.ragged_moe_grouped_ok(ff, D, E) and L.ragged_moe_grouped_ok(D, ff, E)) \
-                or xa.stride(0) % 8 or w_up.shape != (E, ff, D) or w_dn.shape != (E, D, ff) or not w_up.is_contiguous() \
+        if xa.dtype != torch.bfloat16 or not (L.ragged_moe_grouped_ok(wrows, D, E) and L.ragged_moe_grouped_ok(D, ff, E)) \
+                or xa.stride(0) % 8 or w_up.shape != (E, wrows, D) or w_dn.shape != (E, D, ff) or not w_up.is_contiguous() \
                 or not w_dn.is_contiguous() or w_up.dtype != xa.dtype or w_dn.dtype != xa.dtype:
             return None
         _act(xa, w_up, w_dn, base)
@@ -568,7 +584,8 @@ class HipOps:
         A = torch.empty(M, ff, dtype=xa.dtype, device=xa.device)
         ys = torch.empty(M, D, dtype=xa.dtype, device=xa.device)
         _ok(L.ragged_moe_grouped_gemm(xa.data_ptr(), xa.stride(0), src.data_ptr(), w_up.data_ptr(), A.data_ptr(), seg.data_ptr(),
-                                      te.data_ptr(), tr.data_ptr(), nt.data_ptr(), max_tiles, ff, D, E, 1, st), "moe_grouped_gemm (up)")
+                                      te.data_ptr(), tr.data_ptr(), nt.data_ptr(), max_tiles, wrows, D, E, 2 if gated else 1, st),
+            "moe_grouped_gemm (up)")
         _ok(L.ragged_moe_grouped_gemm(A.data_ptr(), ff, None, w_dn.data_ptr(), ys.data_ptr(), seg.data_ptr(), te.data_ptr(),
                                       tr.data_ptr(), nt.data_ptr(), max_tiles, D, ff, E, 0, st), "moe_grouped_gemm (down)")
         return self.moe_combine(ys, place.view(T, top), wts, base)
@@ -588,13 +605,15 @@ class HipOps:
                                      y.data_ptr(), T, D, top, _DT[ys.dtype], _stream()), "moe_combine")
         return y
 
-    def moe_rows(self, xa, idx, wts, w_up, w_dn, base):
-        """y = base + sum over a row's chosen experts of weight * W_down relu(W_up x)^2, every pair served on its own."""
+    def moe_rows(self, xa, idx, wts, w_up, w_dn, base, gated=False):
+        """y = base + sum over a row's chosen experts of weight * W_down relu(W_up x)^2, every pair served on its own.
+        ``gated``: w_up holds (gate, up) rows next to each other and the inner activation is silu(gate) * up."""
         _act(xa, w_up, w_dn, base)
         _f32(wts)
         T, D = xa.shape
-        E, ff, top = w_up.shape[0], w_up.shape[1], idx.shape[1]
-        if w_up.shape != (E, ff, D) or w_dn.shape != (E, D, ff) or not w_up.is_contiguous() or not w_dn.is_contiguous() \
+        E, top = w_up.shape[0], idx.shape[1]
+        ff = w_up.shape[1] // 2 if gated else w_up.shape[1]
+        if w_up.shape != (E, 2 * ff if gated else ff, D) or w_dn.shape != (E, D, ff) or not w_up.is_contiguous() or not w_dn.is_contiguous() \
                 or w_up.dtype != xa.dtype or w_dn.dtype != xa.dtype or idx.shape != (T, top) or wts.shape != (T, top) \
                 or idx.dtype != torch.int32 or not idx.is_contiguous() \
                 or (base is not None and (base.shape != (T, D) or base.dtype != xa.dtype or not base.is_contiguous())):
@@ -603,8 +622,62 @@ class HipOps:
         y = torch.empty(T, D, dtype=xa.dtype, device=xa.device)
         _ok(lib().ragged_moe_rows(xa.data_ptr(), xa.stride(0), idx.data_ptr(), wts.data_ptr(), w_up.data_ptr(), w_dn.data_ptr(),
                                   None if base is None else base.data_ptr(), A.data_ptr(), y.data_ptr(), T, D, ff, top,
-                                  _DT[xa.dtype], _stream()), "moe_rows")
+                                  int(bool(gated)), _DT[xa.dtype], _stream()), "moe_rows")
         return y
+
+    def embed_rows(self, ids, table, ids2=None, table2=None, scale=1.0):
+        """float32 [T, width]: scale * table[ids] (+ table2[ids2]), summed in float."""
+        _act(table, table2)
+        T, D = ids.numel(), table.shape[1]
+        for i, t in ((ids, table), (ids2, table2)):
+            if t is not None and (i is None or i.dtype != torch.int64 or not i.is_contiguous() or i.numel() != T
+                                  or not t.is_contiguous() or t.shape[1] != D or t.dtype != table.dtype or i.device != t.device):
+                raise ValueError("row ids / embedding tables do not fit")
+        x = torch.empty(T, D, dtype=torch.float32, device=table.device)
+        _ok(lib().ragged_embed_rows(ids.data_ptr(), table.data_ptr(), None if table2 is None else ids2.data_ptr(),
+                                    None if table2 is None else table2.data_ptr(), scale, x.data_ptr(), T, D, _DT[table.dtype],
+                                    _stream()), "embed_rows")
+        return x
+
+    def add_norm(self, x, y1, y2, w_next, eps, act):
+        """x <- x + y1 (+ y2) in place on the float32 stream; returns w_next * rmsnorm(x) as ``act`` (None without
+        ``w_next``).  Without y1 it is a plain norm of the stream."""
+        _f32(x, w_next)
+        _act(y1, y2)
+        rows, D = x.shape
+        for y in (y1, y2):
+            if y is not None and (y.shape != x.shape or not y.is_contiguous() or y.dtype != act):
+                raise ValueError("sublayer outputs must match the stream's shape and the activation type")
+        if (y2 is not None and y1 is None) or (w_next is not None and w_next.numel() != D) or not x.is_contiguous():
+            raise ValueError("norm weight / operands do not fit the stream")
+        xa = None if w_next is None else torch.empty(rows, D, dtype=act, device=x.device)
+        _ok(lib().ragged_add_norm(x.data_ptr(), None if y1 is None else y1.data_ptr(), None if y2 is None else y2.data_ptr(),
+                                  None if w_next is None else w_next.data_ptr(), None if xa is None else xa.data_ptr(), rows, D, eps,
+                                  _DT[act], _stream()), "add_norm")
+        return xa
+
+    _ACT_KINDS = {"gelu_erf": 0, "gelu_tanh": 1, "relu2": 2}
+
+    def act_cols(self, P, col0, n, kind):
+        """act(P[:, col0 : col0 + n]) as a contiguous [rows, n] matrix; kind: gelu_erf, gelu_tanh or relu2."""
+        _act(P)
+        if P.dim() != 2 or col0 < 0 or col0 + n > P.shape[1]:
+            raise ValueError("columns outside the matrix")
+        out = torch.empty(P.shape[0], n, dtype=P.dtype, device=P.device)
+        _ok(lib().ragged_act_cols(P.data_ptr(), P.stride(0), col0, out.data_ptr(), P.shape[0], n, self._ACT_KINDS[kind], _DT[P.dtype],
+                                  _stream()), "act_cols")
+        return out
+
+    def glu_pairs(self, P):
+        """silu(P[:, 0::2]) * P[:, 1::2]: inner channels that come as neighbouring (gate, up) pairs."""
+        _act(P)
+        if P.dim() != 2 or P.shape[1] % 2:
+            raise ValueError("(gate, up) pairs expected")
+        out = torch.empty(P.shape[0], P.shape[1] // 2, dtype=P.dtype, device=P.device)
+        if out.numel():
+            _ok(lib().ragged_glu_pairs(P.data_ptr(), P.stride(0), out.data_ptr(), P.shape[0], P.shape[1] // 2, _DT[P.dtype], _stream()),
+                "glu_pairs")
+        return out
 
 
 class TorchOps:
@@ -640,7 +713,7 @@ class TorchOps:
         return out
 
     def conv_head(self, P, col0, meta, *, cw, taps, C, ch0, state, ngroups, gsize, normw, eps, rot, inv_freq,
-                  out_dense=None, pages=None, norm_n=None, rot0=0, interleaved=False):
+                  out_dense=None, pages=None, norm_n=None, rot0=0, interleaved=False, rot_amp=1.0):
         width = ngroups * gsize
         v = self._segment(P, col0, meta, cw, taps, C, ch0, state, width).view(meta.T, ngroups, gsize)
         if normw is not None:
@@ -650,7 +723,7 @@ class TorchOps:
         if rot:
             half = rot // 2
             ang = meta.tok_pos.to(P.device).float()[:, None] * inv_freq[None]
-            c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+            c, s = ang.cos()[:, None, :] * rot_amp, ang.sin()[:, None, :] * rot_amp
             if interleaved:
                 a, b2 = v[..., rot0:rot0 + rot:2], v[..., rot0 + 1:rot0 + rot:2]
                 turned = torch.stack([a * c - b2 * s, b2 * c + a * s], -1).flatten(-2)
@@ -710,7 +783,7 @@ class TorchOps:
         return (v if w is None else v * w).to(act)
 
     def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
-                   eps, gate=None, gate0=0, sink=None):
+                   eps, gate=None, gate0=0, sink=None, chunk=0, softcap=0.0, gate_wide=False):
         out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=q.device)
         q = q.view(meta.T, H, maps, d)
         for b, (slot, past, n, pg) in enumerate(meta.seqs):
@@ -723,11 +796,15 @@ class TorchOps:
             vis = j <= i
             if window > 0:
                 vis &= (i - j < window) | (j < keep_first)
+            if chunk > 0:
+                vis &= (i // chunk) == (j // chunk)
             qs = q[meta.start[b]:meta.start[b] + n]
             rep = H // G
             o = None
             for mp in range(maps):
                 s = torch.einsum("thd,hld->htl", qs[:, :, mp], k[:, :, mp].repeat_interleave(rep, 0)) * scale
+                if softcap > 0:
+                    s = softcap * torch.tanh(s / softcap)
                 s = s.masked_fill(~vis, float("-inf"))
                 if sink is None:
                     w = torch.softmax(s, -1)
@@ -741,7 +818,9 @@ class TorchOps:
             if out_norm:
                 o = o / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)
             out[meta.start[b]:meta.start[b] + n] = (o * out_scale).reshape(n, H * vd)
-        if gate is not None:
+        if gate is not None and gate_wide:
+            out = out * torch.sigmoid(gate[:, gate0:gate0 + H * vd].float())
+        elif gate is not None:
             out = (out.view(meta.T, H, vd) * torch.sigmoid(gate[:, gate0:gate0 + H].float())[:, :, None]).view(meta.T, H * vd)
         return out.to(kpages.dtype)
 
@@ -782,16 +861,20 @@ class TorchOps:
         k = P[:, k0:k0 + H * d].float().view(T, H, d)
         return q, a[:, :, None].expand(T, H, d).reshape(T, -1).contiguous(), (b[:, :, None] * k).reshape(T, -1)
 
-    def moe_route(self, xa, w_router, groups, keep, top, scale):
-        s = torch.softmax(xa.float() @ w_router.t(), -1)
+    def moe_route(self, xa, w_router, groups, keep, top, scale, score="softmax", group_top=1, renorm=False):
+        z = xa.float() @ w_router.t()
+        s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
         E = s.shape[1]
-        best = s.view(-1, groups, E // groups).max(-1).values
+        best = s.view(-1, groups, E // groups).topk(min(group_top, E // groups), -1).values.sum(-1)
         kept = torch.zeros_like(best, dtype=torch.bool)
         kept.scatter_(1, best.topk(keep, -1).indices, True)
         idx = s.masked_fill(~kept.repeat_interleave(E // groups, 1), -1.0).topk(top, -1).indices
-        return idx.to(torch.int32), s.gather(1, idx) * scale
+        w = s.gather(1, idx)
+        if renorm:
+            w = w / (w.sum(-1, keepdim=True) + 1e-20)
+        return idx.to(torch.int32), w * scale
 
-    def moe_sorted(self, xa, idx, wts, w_up, w_dn, base):
+    def moe_sorted(self, xa, idx, wts, w_up, w_dn, base, gated=False):
         return None                                             # (the host statements run the experts one by one)
 
     def moe_combine(self, ys, place, wts, base):
@@ -800,14 +883,39 @@ class TorchOps:
             y += wts[:, j, None] * ys[place[:, j].long()].float()
         return y.to(ys.dtype)
 
-    def moe_rows(self, xa, idx, wts, w_up, w_dn, base):
+    def moe_rows(self, xa, idx, wts, w_up, w_dn, base, gated=False):
         y = torch.zeros(xa.shape[0], w_dn.shape[1]) if base is None else base.float().clone()
         for t in range(xa.shape[0]):
             for j in range(idx.shape[1]):
                 e = int(idx[t, j])
-                a = torch.relu(w_up[e].float() @ xa[t].float()).pow(2).to(xa.dtype)
+                a = w_up[e].float() @ xa[t].float()
+                a = (F.silu(a[0::2]) * a[1::2] if gated else torch.relu(a).pow(2)).to(xa.dtype)
                 y[t] += wts[t, j] * (w_dn[e].float() @ a.float())
         return y.to(xa.dtype)
+
+    def embed_rows(self, ids, table, ids2=None, table2=None, scale=1.0):
+        x = table[ids].float() * scale
+        return x if table2 is None else x + table2[ids2].float()
+
+    def add_norm(self, x, y1, y2, w_next, eps, act):
+        if y1 is not None:
+            x += y1.float() if y2 is None else y1.float() + y2.float()
+        if w_next is None:
+            return None
+        return (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w_next).to(act)
+
+    def act_cols(self, P, col0, n, kind):
+        z = P[:, col0:col0 + n].float()
+        if kind == "gelu_erf":
+            v = 0.5 * z * (1.0 + torch.erf(z * 0.7071067811865476))
+        elif kind == "gelu_tanh":
+            v = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        else:
+            v = torch.relu(z).pow(2)
+        return v.to(P.dtype)
+
+    def glu_pairs(self, P):
+        return (F.silu(P[:, 0::2].float()) * P[:, 1::2].float()).to(P.dtype)
 
 
 def ops_for(device) -> object:
