@@ -84,7 +84,8 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   const int w_lo_last = low_key(w_last, a.window, a.chunk);
   const bool wave_has_rows = 16 * wave < nrows;
   const int my_lo = low_key(qpos, a.window, a.chunk);
-  const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
+  const bool capped = a.softcap > 0.f;
+  const float inv_cap = capped ? 1.0f / a.softcap : 0.f;
 
   const bf16* K = (const bf16*)a.kpages;
   const bf16* V = (const bf16*)a.vpages;
@@ -181,28 +182,20 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
 #pragma unroll
     for (int mp = 0; mp < MAPS; ++mp) {
       float mx = -1e30f;
-      if (inner) {
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
+      for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            S[mp][kb][i] *= a.scale;
-            if (a.softcap > 0.f) S[mp][kb][i] = a.softcap * fast_tanh(S[mp][kb][i] * inv_cap);
-            mx = fmaxf(mx, S[mp][kb][i]);
-          }
-      } else {
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 4; ++i) {
+          float sc = S[mp][kb][i] * a.scale;
+          if (capped) sc = a.softcap * fast_tanh(sc * inv_cap);
+          if (!inner) {
             const int key = k0 + 16 * kb + 4 * g4 + i;
             const bool vis = key <= qpos && (key >= my_lo || key < keep);
-            float sc = S[mp][kb][i] * a.scale;
-            if (a.softcap > 0.f) sc = a.softcap * fast_tanh(sc * inv_cap);
-            S[mp][kb][i] = vis ? sc : -1e30f;
-            mx = fmaxf(mx, S[mp][kb][i]);
+            sc = vis ? sc : -1e30f;
           }
-      }
+          S[mp][kb][i] = sc;
+          mx = fmaxf(mx, sc);
+        }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float mnew = fmaxf(m[mp], mx);

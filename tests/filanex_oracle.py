@@ -75,6 +75,18 @@ def capped(s, cap):
     return cap * torch.tanh(s / cap) if cap else s
 
 
+def attend(q, k, v, scale, cap, size):
+    """q [T, H, d], k [T, G, d], v [T, G, e] -> [T, H, e]: softmax over the visible keys of the capped, scaled scores"""
+    T, H, G = q.shape[0], q.shape[1], k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=F64)
+    for i in range(T):
+        js = [j for j in range(T) if sees(i, j, size)]
+        for h in range(H):
+            g = h // (H // G)
+            out[i, h] = torch.softmax(capped((k[js, g] @ q[i, h]) * scale, cap), 0) @ v[js, g]
+    return out
+
+
 def attention_mixer(u, W, p, m):
     T = u.shape[0]
     H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
@@ -86,14 +98,7 @@ def attention_mixer(u, W, p, m):
         freqs, amp = pair_frequencies(rot)
         q = torch.stack([turn_neighbours(q[t], t, freqs, amp) for t in range(T)])
         k = torch.stack([turn_neighbours(k[t], t, freqs, amp) for t in range(T)])
-    size = (m.get("mask") or {}).get("size")
-    out = torch.zeros(T, H, e, dtype=F64)
-    for i in range(T):
-        js = [j for j in range(T) if sees(i, j, size)]
-        for h in range(H):
-            g = h // (H // G)
-            s = capped((k[js, g] @ q[i, h]) * m["scale"], m.get("softcap"))
-            out[i, h] = torch.softmax(s, 0) @ v[js, g]
+    out = attend(q, k, v, m["scale"], m.get("softcap"), (m.get("mask") or {}).get("size"))
     gate = torch.sigmoid(u @ W[p + "g"].T)
     return (out.reshape(T, H * e) * gate) @ W[p + "o"].T
 
@@ -175,3 +180,78 @@ def forward(tokens, W, config, collect=None, choices=None):
         if collect is not None:
             collect.append(x.clone())
     return norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+# ---------------------------------------------------------------------------------------- small models for the tests
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, size=24, cap=8.0, scale=None, rot=(8, 500.0, (3.0, 64, 4.0, 0.5)),
+                    mlp="dense"):
+    """rot: (dims, base, scaling or None) with scaling = (factor, original, fast, slow); None: no rotation"""
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale or 2.0 * dim ** -0.5}
+    if size:
+        m["mask"] = {"size": size}
+    if cap:
+        m["softcap"] = cap
+    if rot:
+        m["rot"] = {"dims": rot[0], "base": rot[1]}
+        if rot[2]:
+            m["rot"]["scaling"] = dict(zip(("factor", "original", "fast", "slow"), rot[2]))
+    return {"type": "attention", "mixer": m, "mlp": dense(40) if mlp == "dense" else mlp}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts=6, top=2, ff=12, count=3, keep=2):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "groups": {"count": count, "keep": keep}}}
+
+
+def make_config(layers, vocab=80, width=48, loop=None, pairs=(37, 11, 5), eps=1e-5):
+    """loop: (start, stop, times) or None; pairs: (buckets, mul_prev, mul_cur) or None"""
+    cfg = {"architecture": "Filanex", "layers": layers, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+    if pairs:
+        cfg["embedding"] = {"bigram": dict(zip(("buckets", "mul_prev", "mul_cur"), pairs))}
+    if loop:
+        cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return cfg
+
+
+def random_weights(config, seed=0):
+    """bfloat16 checkpoint tensors; router rows are wide enough that the choices vary from token to token"""
+    g = torch.Generator().manual_seed(seed)
+    D = config["width"]
+
+    def mat(n, k, s=1.0):
+        return (torch.randn(n, k, generator=g) * (s / math.sqrt(k))).to(torch.bfloat16)
+
+    def vec(n, mean=0.0, s=0.1):
+        return (mean + s * torch.randn(n, generator=g)).to(torch.bfloat16)
+
+    sd = {"embed": mat(config["vocab"], D, math.sqrt(D)), "final.norm": vec(D, 1.0), "head": mat(config["vocab"], D)}
+    table = (config.get("embedding") or {}).get("bigram")
+    if table:
+        sd["bigram"] = mat(table["buckets"] + 1, D, math.sqrt(D))
+    if config.get("loop"):
+        sd["loop.in"] = mat(D, 2 * D, 1.4)
+    for li, spec in enumerate(config["layers"]):
+        p, q, m = f"l{li}.mix.", f"l{li}.mlp.", spec["mixer"]
+        H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        sd[f"l{li}.norm1"] = vec(D, 1.0, 0.2)
+        sd[p + "q"], sd[p + "k"], sd[p + "v"], sd[p + "g"] = mat(H * d, D, 2.0), mat(G * d, D, 2.0), mat(G * e, D), mat(H * e, D, 2.0)
+        sd[p + "o"] = mat(D, H * e)
+        f = spec.get("mlp")
+        if f is None:
+            continue
+        if f["kind"] == "dense":
+            sd[q + "up"], sd[q + "up.b"] = mat(f["ff"], D), vec(f["ff"], 0.0, 0.3)
+            sd[q + "down"], sd[q + "down.b"] = mat(D, f["ff"]), vec(D, 0.0, 0.3)
+        else:
+            sd[q + "router"] = mat(f["router"]["experts"], D, 3.0)
+            for x in range(f["router"]["experts"]):
+                n = f["expert"]["ff"]
+                sd[q + f"e{x}.gate"], sd[q + f"e{x}.up"], sd[q + f"e{x}.down"] = mat(n, D, 2.0), mat(n, D), mat(D, n)
+    return sd
+
+
+def as_f64(sd):
+    return {k: v.double() for k, v in sd.items()}

@@ -151,8 +151,10 @@ def test_unequal_requests_in_one_batch_and_reuse_of_pages_and_slots(device, dens
     old, new = ("a", "b", "c"), ("d", "e", "f")
     assert set().union(*(seen[k][0] for k in new)) & set().union(*(seen[k][0] for k in old)), "no page was used twice"
     assert set().union(*(seen[k][1] for k in new)) & set().union(*(seen[k][1] for k in old)), "no slot was used twice"
-    alone = run_schedule(eng, {"c": prompts["c"]}, [[("c", 70)]], 128)["c"]          # alone as inside the batch
-    close(alone, got["c"], 1e-4)
+    # alone as inside the batch: the library's products sum in an order that depends on their row count, so the two
+    # differ by rounding (each is within F32_TOL of the float64 statement)
+    alone = run_schedule(eng, {"c": prompts["c"]}, [[("c", 70)]], 128)["c"]
+    close(alone, got["c"], 2e-4)
 
 
 @pytest.mark.parametrize("device", DEVICES)
