@@ -44,10 +44,27 @@ def build(force: bool = False) -> Path:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     _LIB_PATH.parent.mkdir(exist_ok=True)
     tmp = _LIB_PATH.with_suffix(f".{os.getpid()}.tmp")
-    cmd = [hipcc, *HIP_FLAGS, "-shared", "-o", str(tmp), *map(str, srcs)]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)
+    # the translation units are compiled side by side (one hipcc each), then linked
+    objs = [_LIB_PATH.parent / f".ragged_{os.getpid()}_{p.stem}.o" for p in srcs]
+    procs = [(subprocess.Popen([hipcc, *HIP_FLAGS, "-c", "-o", str(o), str(p)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                               text=True), p) for p, o in zip(srcs, objs)]
+    failed = []
+    for proc, p in procs:
+        out, _ = proc.communicate()
+        if proc.returncode != 0:
+            failed.append(f"{p}:\n{out}")
+    try:
+        if not failed:
+            cmd = [hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", str(tmp), *map(str, objs)]
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                failed.append(" ".join(cmd) + "\n" + r.stdout + r.stderr)
+    finally:
+        for o in objs:
+            if o.exists():
+                o.unlink()
+    if failed:
+        sys.stderr.write("\n".join(failed))
         raise RuntimeError("building libbigdl_ragged.so failed")
     os.replace(tmp, _LIB_PATH)
     return _LIB_PATH
