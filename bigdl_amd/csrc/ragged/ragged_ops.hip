@@ -619,19 +619,32 @@ extern "C" int ragged_add_norm(float* x, const void* y1, const void* y2, const f
 // Activations of a feed-forward's inner channels.  act_cols: out[r, c] = act(P[r, col0 + c]), c < n, with
 // kind 0: gelu through erf, 0.5 z (1 + erf(z / sqrt 2));  1: gelu through tanh, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)));
 // 2: relu(z)^2.  glu_pairs: the inner channels come as neighbouring (gate, up) pairs, out[r, c] = silu(P[r, 2 c]) * P[r, 2 c + 1].
-template <typename T>
-__global__ __launch_bounds__(256) void act_cols_kernel(const T* __restrict__ P, int64_t ldp, int col0, T* __restrict__ out, int64_t rows,
-                                                       int n, int kind) {
-  const int64_t total = rows * n;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    const int64_t r = i / n;
-    const int c = (int)(i % n);
-    const float z = to_f(P[r * ldp + col0 + c]);
-    float v;
-    if (kind == 0) v = 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
-    else if (kind == 1) v = 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
-    else { v = fmaxf(z, 0.f); v *= v; }
-    out[i] = from_f<T>(v);
+__device__ __forceinline__ float act_value(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+  if (kind == 1) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+  const float v = fmaxf(z, 0.f);
+  return v * v;
+}
+
+// grid (blocks of 256 pieces of a row, rows); VEC: a thread takes 16 bytes of a row (rows and the first column are
+// 16-byte aligned, n a multiple of the piece), otherwise one element
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void act_cols_kernel(const T* __restrict__ P, int64_t ldp, int col0, T* __restrict__ out, int n,
+                                                       int kind) {
+  constexpr int N = VEC ? 16 / (int)sizeof(T) : 1;
+  const int64_t r = blockIdx.y;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * N;
+  if (c >= n) return;
+  const T* src = P + r * ldp + col0 + c;
+  T* dst = out + r * n + c;
+  if (VEC) {
+    union { uint4 q; T e[N]; } v;
+    v.q = *reinterpret_cast<const uint4*>(src);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v.e[i] = from_f<T>(act_value(to_f(v.e[i]), kind));
+    *reinterpret_cast<uint4*>(dst) = v.q;
+  } else {
+    dst[0] = from_f<T>(act_value(to_f(src[0]), kind));
   }
 }
 
@@ -648,11 +661,18 @@ __global__ __launch_bounds__(256) void glu_pairs_kernel(const T* __restrict__ P,
 
 extern "C" int ragged_act_cols(const void* P, int64_t ldp, int col0, void* out, int64_t rows, int n, int kind, int dtype,
                                hipStream_t st) {
-  if (rows <= 0 || n <= 0 || col0 < 0 || ldp < col0 + n || kind < 0 || kind > 2) return -1;
-  const int64_t blocks = (rows * n + 255) / 256;
-  const unsigned grid = (unsigned)(blocks < 16384 ? blocks : 16384);
-  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((act_cols_kernel<T>), dim3(grid), dim3(256), 0, st, (const T*)P, ldp, col0, (T*)out, rows, n,
-                                            kind))
+  if (rows <= 0 || rows > 65535LL * 65535LL || n <= 0 || col0 < 0 || ldp < col0 + n || kind < 0 || kind > 2) return -1;
+  RAGGED_DISPATCH(dtype,
+    constexpr int N = 16 / (int)sizeof(T);
+    const bool vec = n % N == 0 && ldp % N == 0 && col0 % N == 0 && ((uintptr_t)P % 16) == 0 && ((uintptr_t)out % 16) == 0;
+    // (the grid's second dimension holds at most 65535 rows: more rows go in several launches)
+    for (int64_t r0 = 0; r0 < rows; r0 += 65535) {
+      const unsigned nr = (unsigned)(rows - r0 < 65535 ? rows - r0 : 65535);
+      const T* src = (const T*)P + r0 * ldp;
+      T* dst = (T*)out + r0 * n;
+      if (vec) hipLaunchKernelGGL((act_cols_kernel<T, true>), dim3((n / N + 255) / 256, nr), dim3(256), 0, st, src, ldp, col0, dst, n, kind);
+      else hipLaunchKernelGGL((act_cols_kernel<T, false>), dim3((n + 255) / 256, nr), dim3(256), 0, st, src, ldp, col0, dst, n, kind);
+    })
   return RAGGED_LAUNCH_OK();
 }
 

@@ -374,11 +374,15 @@ def test_embedding_sum_stream_update_and_activations(device):
     i1, i2 = torch.randint(0, 20, (33,), generator=g), torch.randint(0, 9, (33,), generator=g)
     close(ops.embed_rows(i1.to(device), t1.to(device), i2.to(device), t2.to(device), 1.0).double().cpu(), t1[i1].double() + t2[i2].double(), 1e-6)
     close(ops.embed_rows(i1.to(device), t1.to(device), scale=3.0).double().cpu(), 3.0 * t1[i1].double(), 1e-5)
-    P = torch.randn(11, 50, generator=g) * 3
-    z = P[:, 7:47].double()
-    close(ops.act_cols(P.to(device), 7, 40, "gelu_erf").double().cpu(), 0.5 * z * (1 + torch.erf(z / math.sqrt(2))), 1e-5)
-    close(ops.act_cols(P.to(device), 7, 40, "gelu_tanh").double().cpu(),
-          0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3))), 1e-5)
+    for width, c0, n in ((50, 7, 40), (56, 8, 40), (1040, 16, 1024)):      # columns that are and are not 16-byte pieces
+        P = torch.randn(11, width, generator=g) * 3
+        z = P[:, c0:c0 + n].double()
+        close(ops.act_cols(P.to(device), c0, n, "gelu_erf").double().cpu(), 0.5 * z * (1 + torch.erf(z / math.sqrt(2))), 1e-5)
+        close(ops.act_cols(P.to(device), c0, n, "gelu_tanh").double().cpu(),
+              0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3))), 1e-5)
+        Pb = P.bfloat16()
+        zb = Pb[:, c0:c0 + n].double()
+        close(ops.act_cols(Pb.to(device), c0, n, "gelu_erf").double().cpu(), 0.5 * zb * (1 + torch.erf(zb / math.sqrt(2))), 0.05)
 
 
 def test_pair_rows_continue_across_steps_and_start_anew_in_a_used_slot():
@@ -456,6 +460,30 @@ def test_greedy_generation_through_the_auto_class_and_the_scheduler(device, tmp_
     assert cb.mixed_steps > 0 and not cb.pool.len_of and len(cb.pool.free_pages) == cb.pool.num_pages
     for r in reqs:
         _greedy_is_consistent(cfg, W, r.input_ids + r.output_ids, len(r.input_ids))
+
+
+def test_command_line_and_sampling(tmp_path, capsys):
+    """``llm-cli --prompt-ids`` on a checkpoint without a tokenizer (greedy), and sampled generation through the same
+    scheduler: with a fixed seed it repeats itself, and top_k = 1 is the greedy answer"""
+    from bigdl_amd.cli import llm_cli
+    from bigdl_amd.transformers import AutoModelForCausalLM
+    cfg = O.make_config([O.attention_layer(), O.attention_layer(mlp=O.moe())], loop=(0, 2, 2))
+    sd = O.random_weights(cfg, seed=91)
+    path = _save_checkpoint(tmp_path, cfg, sd)
+    prompt = tokens(11, cfg["vocab"], 92)
+    model = AutoModelForCausalLM.from_pretrained(path).to("cpu", torch.float32)
+    greedy = model.generate(torch.tensor([prompt]), max_new_tokens=7)[0].tolist()
+    _greedy_is_consistent(cfg, O.as_f64(sd), greedy, len(prompt))
+    assert model.generate(torch.tensor([prompt]), max_new_tokens=7, do_sample=True, top_k=1)[0].tolist() == greedy
+    torch.manual_seed(3)
+    a = model.generate(torch.tensor([prompt]), max_new_tokens=7, do_sample=True, temperature=1.5)[0].tolist()
+    torch.manual_seed(3)
+    assert model.generate(torch.tensor([prompt]), max_new_tokens=7, do_sample=True, temperature=1.5)[0].tolist() == a
+    if torch.cuda.is_available():
+        return                                               # (the command line would take the GPU: covered by the gpu tests)
+    served = AutoModelForCausalLM.from_pretrained(path).to("cpu").generate(torch.tensor([prompt]), max_new_tokens=7)[0].tolist()
+    llm_cli.main(["-m", path, "--prompt-ids", " ".join(map(str, prompt)), "-n", "7"])     # (the default type: bfloat16)
+    assert capsys.readouterr().out.split()[-7:] == [str(t) for t in served[len(prompt):]]
 
 
 def test_trace_runner_replays_steps(tmp_path):
