@@ -4,7 +4,7 @@
   bigdl_amd/lib/libbigdl_hip.so    hipcc --offload-arch=gfx950  (all device kernels + decode engine)
   bigdl_amd/lib/libbigdl_ragged.so hipcc --offload-arch=gfx950  (csrc/ragged: the kernels of the ragged engine; a library
                                    of its own so that a checkout without built files that only serves such a model
-                                   compiles two translation units, see ops/ragged.py::build)
+                                   compiles only these few translation units, see ops/ragged.py::build)
 
 Both expose a plain C ABI and are loaded with ctypes, so neither needs the PyTorch
 headers: a full rebuild is a few seconds per file and hipcc cross-compiles gfx950

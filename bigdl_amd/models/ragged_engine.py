@@ -9,7 +9,7 @@ into arbitrary portions next to single decoded tokens run here instead:
   product runs once over all rows; the mixers read ``BatchMeta`` (row -> sequence, position, pages);
 * keys / values live in 64-token pages of a ``PagedStatePool``, per-sequence state in its slots;
 * the mixers are described by small dataclasses whose fields are the design's constants, so a new design is a new list
-  of them (``models/lipizen.py`` and ``models/merusun.py`` build one from a ``config.json``);
+  of them (``models/lipizen.py``, ``models/merusun.py`` and ``models/filanex.py`` build one from a ``config.json``);
 * three residual forms: the post-sum norm x <- norm(alpha x + f(x)), the sandwich x <- x + norm_b(f(norm_a(x))), and the
   parallel pre-norm block u = norm(x), x <- x + mixer(u) + ff(u);
 * a run of layers may be executed several times with the same weights (every execution has its own cache), with the
