@@ -30,6 +30,9 @@ struct AttnArgs {
                          // is visible from i only inside i's block (on top of j <= i and of the window, if any)
   float softcap;         // > 0: scores pass through softcap * tanh(score / softcap) after the scale
   int gate_wide;         // 1: one gate logit per output channel (column gate0 + h * vd + c) instead of one per head
+  const float* sinks;    // [H] or null: with `sink`, head h's own sink score instead of sink_score
+  const float* slopes;   // [H] or null: slopes[h] * (i - j) is taken off the scaled score of query i and key j (in front of
+                         // the cap, if there is one): a bias that grows with the distance
 };
 
 namespace ragged {

@@ -194,6 +194,13 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
 #pragma unroll
         for (int mp = 0; mp < MAPS; ++mp) s[r][mp] *= a.scale;
     }
+    if (a.slopes) {
+      const float dist = (float)(i - kp);
+#pragma unroll
+      for (int r = 0; r < REP; ++r)
+#pragma unroll
+        for (int mp = 0; mp < MAPS; ++mp) s[r][mp] -= a.slopes[h0 + r] * dist;
+    }
     if (a.softcap > 0.f) {
       const float inv_cap = 1.0f / a.softcap;
 #pragma unroll
@@ -277,12 +284,13 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
     for (int mp = 0; mp < MAPS; ++mp) {
       float M = -1e30f, L = 0.f, w[8];
       for (int wv = 0; wv < nw; ++wv) M = fmaxf(M, part0[wv * wstride + r * pstride + mp]);
-      if (a.sink) M = fmaxf(M, a.sink_score);
+      const float sink_score = a.sinks ? a.sinks[h] : a.sink_score;
+      if (a.sink) M = fmaxf(M, sink_score);
       for (int wv = 0; wv < nw; ++wv) {
         w[wv] = __expf(part0[wv * wstride + r * pstride + mp] - M);
         L += w[wv] * part0[wv * wstride + r * pstride + MAPS + mp];
       }
-      if (a.sink) L += __expf(a.sink_score - M);
+      if (a.sink) L += __expf(sink_score - M);
       const float coef = (mp == 0 ? 1.0f : -a.lambda) / L;
 #pragma unroll
       for (int v = 0; v < VRP; ++v) {
@@ -371,7 +379,7 @@ static void launch_rows(AttnArgs a, Batch bt, int nrows, hipStream_t st, int* rc
 
 extern "C" int ragged_paged_attn(AttnArgs a, Batch bt, int maps, int dtype, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || a.d <= 0 || a.vd <= 0 || a.vd > 128 * MAX_VRP) return -1;
-  if ((maps != 1 && maps != 2) || a.ldv < a.vd || a.chunk < 0 || (a.gate_wide && !a.gate)) return -1;
+  if ((maps != 1 && maps != 2) || a.ldv < a.vd || a.chunk < 0 || (a.gate_wide && !a.gate) || (a.sinks && !a.sink)) return -1;
   const int nrows = a.rows ? a.n_rows : bt.T;
   if (nrows <= 0 || (int64_t)nrows * a.H > 0x7fffffff) return -1;
   int rc = 0;

@@ -86,6 +86,8 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   const int my_lo = low_key(qpos, a.window, a.chunk);
   const bool capped = a.softcap > 0.f;
   const float inv_cap = capped ? 1.0f / a.softcap : 0.f;
+  const bool biased = a.slopes != nullptr;                   // scores fall with the distance between query and key
+  const float slope = biased ? a.slopes[h] : 0.f;
 
   const bf16* K = (const bf16*)a.kpages;
   const bf16* V = (const bf16*)a.vpages;
@@ -187,6 +189,7 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           float sc = S[mp][kb][i] * a.scale;
+          if (biased) sc -= slope * (float)(qpos - (k0 + 16 * kb + 4 * g4 + i));
           if (capped) sc = a.softcap * fast_tanh(sc * inv_cap);
           if (!inner) {
             const int key = k0 + 16 * kb + 4 * g4 + i;
@@ -244,10 +247,11 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   if (!rowok) return;
   // ---- epilogue: combine the maps, per-head norm, gate; the lane holds channels 16 eb + 4 g4 + i of its query
   if (a.sink) {                                              // one more term in every normaliser
+    const float sink_score = a.sinks ? a.sinks[h] : a.sink_score;
 #pragma unroll
     for (int mp = 0; mp < MAPS; ++mp) {
-      const float mnew = fmaxf(m[mp], a.sink_score), corr = __expf(m[mp] - mnew);
-      l[mp] = l[mp] * corr + __expf(a.sink_score - mnew);
+      const float mnew = fmaxf(m[mp], sink_score), corr = __expf(m[mp] - mnew);
+      l[mp] = l[mp] * corr + __expf(sink_score - mnew);
 #pragma unroll
       for (int eb = 0; eb < MF_NEB; ++eb) O[mp][eb] *= corr;
     }
@@ -497,7 +501,7 @@ static int launch_wide(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
 
 extern "C" int ragged_paged_attn_mfma_wide(AttnArgs a, Batch bt, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_wide_ok(a.d, a.vd)) return -1;
-  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate || a.chunk > 0 || a.softcap > 0.f) return -1;
+  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate || a.chunk > 0 || a.softcap > 0.f || a.sinks || a.slopes) return -1;
   if (!a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
   const unsigned grid = (unsigned)(a.n_tiles * a.H);
   const int dk = (a.d + 31) / 32, neb = a.vd / 16;
@@ -693,7 +697,7 @@ static int launch_heads(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
 // token rows a.rows[0 .. n_rows) (all T rows without a list)
 extern "C" int ragged_paged_attn_mfma_heads(AttnArgs a, Batch bt, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_wide_ok(a.d, a.vd)) return -1;
-  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate || a.chunk > 0 || a.softcap > 0.f) return -1;
+  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate || a.chunk > 0 || a.softcap > 0.f || a.sinks || a.slopes) return -1;
   const int nrows = a.rows ? a.n_rows : bt.T;
   const int nblk = (a.H / a.G + 15) / 16;
   if (nrows <= 0 || (int64_t)nrows * a.G * nblk > 0x7fffffff) return -1;
@@ -727,7 +731,7 @@ extern "C" int ragged_paged_attn_mfma(AttnArgs a, Batch bt, int maps, hipStream_
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_ok(a.d, a.vd)) return -1;
   if (a.ldv < a.vd || a.ldv % 8) return -1;                  // value rows are read 16 bytes at a time
   // per-channel gate logits are read 8 bytes at a time
-  if (a.chunk < 0 || (a.gate_wide && (!a.gate || a.ldg % 4 || a.gate0 % 4))) return -1;
+  if (a.chunk < 0 || (a.gate_wide && (!a.gate || a.ldg % 4 || a.gate0 % 4)) || (a.sinks && !a.sink)) return -1;
   if ((maps != 1 && maps != 2) || !a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
   const unsigned grid = (unsigned)(a.n_tiles * a.H);
   if (maps == 2) launch_mfma<2>(a, bt, grid, st);

@@ -1,0 +1,204 @@
+// Generalised delta rule of the ragged engine: a matrix state per head that decays per key channel, forgets along the
+// direction of the unit key and then takes the new key / value pair,
+//     S_t = diag(w_t) S_(t-1) - (a_t * n_t) (n_t^T S_(t-1)) + k_t v_t^T,     o_t = S_t^T r_t,     n = k / sqrt(|k|^2 + tiny)
+// with both terms reading the old state.  S float [d, vd] per (slot, head).  Everything but the projections themselves
+// (decay, removal rate, unit key, state, outputs) is float whatever the activation type T is.
+#include "ragged_common.h"
+
+using namespace ragged;
+
+// ---------------------------------------------------------------------------------------------------------------
+// The scan's five arrays from this step's projections, float [rows, H d] each:
+//   rf = r,  wf = exp(-rate * sigmoid(decay logits + w0)),  nf = n,  bf = sigmoid(a logits + ab) * n,  kf = k
+// r, k and the a logits are columns of P (type T); the decay logits come from a second small product and are float.
+// One wavefront per (row, head).
+template <typename T>
+__global__ __launch_bounds__(256) void delta_gates_kernel(const T* __restrict__ P, int64_t ldp, int r0, int k0, int a0,
+                                                          const float* __restrict__ wl, const float* __restrict__ w0,
+                                                          const float* __restrict__ ab, float rate, float tiny,
+                                                          float* __restrict__ rf, float* __restrict__ wf, float* __restrict__ nf,
+                                                          float* __restrict__ bf, float* __restrict__ kf, int64_t items, int H, int d) {
+  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (item >= items) return;
+  const int64_t t = item / H;
+  const int h = (int)(item % H);
+  const T* row = P + t * ldp;
+  float ss = 0.f;
+  for (int c = lane; c < d; c += 64) { const float k = to_f(row[k0 + h * d + c]); ss += k * k; }
+  const float inv = 1.0f / sqrtf(wave_sum(ss) + tiny);
+  for (int c = lane; c < d; c += 64) {
+    const int ch = h * d + c;
+    const int64_t o = t * (int64_t)(H * d) + ch;
+    const float k = to_f(row[k0 + ch]), n = k * inv;
+    const float sw = 1.0f / (1.0f + expf(-(wl[o] + w0[ch])));
+    const float sa = 1.0f / (1.0f + expf(-(to_f(row[a0 + ch]) + ab[ch])));
+    rf[o] = to_f(row[r0 + ch]);
+    wf[o] = expf(-rate * sw);
+    nf[o] = n;
+    bf[o] = sa * n;
+    kf[o] = k;
+  }
+}
+
+extern "C" int ragged_delta_gates(const void* P, int64_t ldp, int r0, int k0, int a0, const float* wl, const float* w0,
+                                  const float* ab, float rate, float tiny, float* rf, float* wf, float* nf, float* bf, float* kf,
+                                  int64_t rows, int H, int d, int dtype, hipStream_t st) {
+  if (rows <= 0 || H <= 0 || d <= 0 || rows * H > 0x7fffffff || r0 < 0 || k0 < 0 || a0 < 0) return -1;
+  const int64_t items = rows * H;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((delta_gates_kernel<T>), dim3((unsigned)((items + 3) / 4)), dim3(256), 0, st, (const T*)P,
+                                            ldp, r0, k0, a0, wl, w0, ab, rate, tiny, rf, wf, nf, bf, kf, items, H, d))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The scan.  Columns of S are independent: column j follows s <- w * s - b (n . s) + k v_j, and its output is r . s.
+// A wavefront owns 64 / R columns; R neighbouring lanes share a column, lane r of them holds rows 32 r .. 32 r + 31 in
+// registers (R = d / 32 rounded up to a power of two; rows past d carry w = 1 and zeros and stay zero), so a token costs
+// two cross-lane sums of R partial products (DPP moves): n . s before the update, r . s after it.  A workgroup is four such
+// wavefronts.  The five arrays of a block of TB tokens are brought into LDS by the whole workgroup with coalesced loads
+// while the previous block is scanned (register look-ahead, two LDS buffers) and read back as 16-byte broadcasts.
+// Grid: (column blocks, heads, sequences).  `values` = 0: v is taken as 0 (the state only decays and forgets: from an
+// identity state this yields a chunk's transition matrix).
+constexpr int DL_DR = 32;
+constexpr int DL_SEG = DL_DR + 4;   // LDS floats per lane group and token (padding shifts the banks between groups)
+constexpr int DL_TBR = 32;          // TB * R <= this
+constexpr int DL_NA = 5;
+constexpr int DL_PRE = DL_NA * DL_TBR * DL_DR / 256;
+
+template <typename T>
+__global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ rf, const float* __restrict__ wf,
+                                                         const float* __restrict__ nf, const float* __restrict__ bf,
+                                                         const float* __restrict__ kf, const T* __restrict__ P, int64_t ldp, int v0,
+                                                         float* __restrict__ state, float* __restrict__ out, int H, int d, int vd,
+                                                         int R, int TB, int values, Batch bt) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 x { r, w, n, b, k: [TB][R][SEG] each, v[TB][wcols] }
+  const int b = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int cols = 64 / R, wcols = 4 * cols;
+  const int r = lane % R, lc = wave * cols + lane / R;     // column inside the workgroup's block
+  const int col = blockIdx.x * wcols + lc;
+  const int start = bt.seq_start[b], n = bt.seq_start[b + 1] - start, past = bt.seq_past[b], slot = bt.seq_slot[b];
+  const bool colok = col < vd;
+  const int row0 = r * DL_DR;
+  const int HD = H * d;
+  const int qsz = TB * R * DL_SEG;                         // floats of one array in a buffer
+  const int bufsz = DL_NA * qsz + TB * wcols;
+  float S[DL_DR];
+  float* sp = state + (((int64_t)slot * H + h) * d) * vd;
+  {
+    const int cc = colok ? col : vd - 1;
+#pragma unroll
+    for (int k = 0; k < DL_DR; ++k) {
+      const int row = row0 + k;
+      const float v = sp[(int64_t)(row < d ? row : d - 1) * vd + cc];    // no condition around the load
+      S[k] = (past > 0 && colok && row < d) ? v : 0.f;
+    }
+  }
+  float pre[DL_PRE], prev[4];
+  const int nel = TB * R * DL_DR;                          // elements of one array in a block, padded rows included
+  auto fetch = [&](int i0) {                               // block of tokens i0 .. i0 + TB - 1 into registers
+#pragma unroll
+    for (int u = 0; u < DL_PRE; ++u) {
+      const int e = tid + 256 * u;
+      const int which = e / nel, rem = e - which * nel;
+      const int tk = rem / (R * DL_DR), row = rem % (R * DL_DR);
+      float v = which == 1 ? 1.f : 0.f;                    // padding: w = 1, everything else 0
+      if (e < DL_NA * nel && row < d && i0 + tk < n) {
+        const float* src = which == 0 ? rf : which == 1 ? wf : which == 2 ? nf : which == 3 ? bf : kf;
+        v = src[(int64_t)(start + i0 + tk) * HD + h * d + row];
+      }
+      pre[u] = v;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = tid + 256 * u;
+      float v = 0.f;
+      if (e < TB * wcols && values) {
+        const int tk = e / wcols, c = blockIdx.x * wcols + e % wcols;
+        if (i0 + tk < n && c < vd) v = to_f(P[(int64_t)(start + i0 + tk) * ldp + v0 + h * vd + c]);
+      }
+      prev[u] = v;
+    }
+  };
+  auto stash = [&](float* buf) {
+#pragma unroll
+    for (int u = 0; u < DL_PRE; ++u) {
+      const int e = tid + 256 * u;
+      if (e < DL_NA * nel) {
+        const int which = e / nel, rem = e - which * nel;
+        const int tk = rem / (R * DL_DR), row = rem % (R * DL_DR);
+        buf[which * qsz + (tk * R + row / DL_DR) * DL_SEG + row % DL_DR] = pre[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = tid + 256 * u;
+      if (e < TB * wcols) buf[DL_NA * qsz + e] = prev[u];
+    }
+  };
+  if (n > 0) { fetch(0); stash(smem); }
+  __syncthreads();
+  int cur = 0;
+  for (int i0 = 0; i0 < n; i0 += TB) {
+    const bool more = i0 + TB < n;
+    if (more) fetch(i0 + TB);
+    const float* buf = smem + cur * bufsz;
+    const int nt = n - i0 < TB ? n - i0 : TB;
+    for (int tk = 0; tk < nt; ++tk) {
+      const int seg = (tk * R + r) * DL_SEG;
+      const float4* r4 = reinterpret_cast<const float4*>(buf + seg);
+      const float4* w4 = reinterpret_cast<const float4*>(buf + qsz + seg);
+      const float4* n4 = reinterpret_cast<const float4*>(buf + 2 * qsz + seg);
+      const float4* b4 = reinterpret_cast<const float4*>(buf + 3 * qsz + seg);
+      const float4* k4 = reinterpret_cast<const float4*>(buf + 4 * qsz + seg);
+      const float v = buf[DL_NA * qsz + tk * wcols + lc];
+      // n . s over the old state
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < DL_DR / 4; ++k) {
+        const float4 a = n4[k];
+        acc[0] += S[4 * k] * a.x; acc[1] += S[4 * k + 1] * a.y; acc[2] += S[4 * k + 2] * a.z; acc[3] += S[4 * k + 3] * a.w;
+      }
+      const float dot = group_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), R);
+      acc[0] = acc[1] = acc[2] = acc[3] = 0.f;
+#pragma unroll
+      for (int k = 0; k < DL_DR / 4; ++k) {
+        const float4 w = w4[k], bb = b4[k], kk = k4[k], q = r4[k];
+        S[4 * k] = w.x * S[4 * k] - bb.x * dot + kk.x * v;
+        S[4 * k + 1] = w.y * S[4 * k + 1] - bb.y * dot + kk.y * v;
+        S[4 * k + 2] = w.z * S[4 * k + 2] - bb.z * dot + kk.z * v;
+        S[4 * k + 3] = w.w * S[4 * k + 3] - bb.w * dot + kk.w * v;
+        acc[0] += S[4 * k] * q.x; acc[1] += S[4 * k + 1] * q.y; acc[2] += S[4 * k + 2] * q.z; acc[3] += S[4 * k + 3] * q.w;
+      }
+      const float tot = group_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), R);
+      if (out && r == 0 && colok) out[(int64_t)(start + i0 + tk) * (H * vd) + h * vd + col] = tot;
+    }
+    if (more) stash(smem + (cur ^ 1) * bufsz);
+    __syncthreads();
+    cur ^= 1;
+  }
+#pragma unroll
+  for (int k = 0; k < DL_DR; ++k) {
+    const int row = row0 + k;
+    if (colok && row < d) sp[(int64_t)row * vd + col] = S[k];
+  }
+}
+
+// out may be null (only the end states are wanted); values = 0: the value columns of P are not read and count as 0
+extern "C" int ragged_delta_scan(const float* rf, const float* wf, const float* nf, const float* bf, const float* kf, const void* P,
+                                 int64_t ldp, int v0, float* state, float* out, int H, int d, int vd, int values, Batch bt,
+                                 int dtype, hipStream_t st) {
+  if (bt.B <= 0 || H <= 0 || d <= 0 || vd <= 0 || d > DL_DR * 32 || (values && !P)) return -1;
+  int R = 1;
+  while (R * DL_DR < d) R <<= 1;
+  const int wcols = 4 * (64 / R);
+  int TB = DL_TBR / R < 16 ? DL_TBR / R : 16;
+  if (TB * wcols > 4 * 256) TB = 4 * 256 / wcols;           // the value look-ahead holds 4 floats per thread
+  if (TB < 1) return -1;
+  const size_t sm = 2 * (size_t)(DL_NA * TB * R * DL_SEG + TB * wcols) * sizeof(float);
+  const dim3 grid((vd + wcols - 1) / wcols, H, bt.B);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((delta_scan_kernel<T>), grid, dim3(256), sm, st, rf, wf, nf, bf, kf, (const T*)P, ldp, v0,
+                                            state, out, H, d, vd, R, TB, values, bt))
+  return RAGGED_LAUNCH_OK();
+}

@@ -94,13 +94,13 @@ extern "C" int ragged_mlstm_expand(const void* P, int64_t ldp, int q0, int k0, c
 }
 
 // out[t, h, :] = u / rms(u) * w[h, :] * sigmoid(gate logits of row t, columns g0 + h * vd ...), u = o[t, h, :vd], or with
-// `em`: u = o[t, h, :vd] / (max(|o[t, h, vd]|, em[t, h]) + floor).  o has ldo floats per (row, head).
-// One wavefront per (row, head).
+// `em`: u = o[t, h, :vd] / (max(|o[t, h, vd]|, em[t, h]) + floor).  o has ldo floats per (row, head).  `scale` multiplies the
+// result (a mixer that is one of two summed side by side carries its weight here).  One wavefront per (row, head).
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                                              const T* __restrict__ P, int64_t ldp, int g0, T* __restrict__ out,
                                                              int64_t items, int H, int vd, float eps, int ldo,
-                                                             const float* __restrict__ em, float den_floor) {
+                                                             const float* __restrict__ em, float den_floor, float scale) {
   const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (item >= items) return;
@@ -112,18 +112,18 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   for (int c = lane; c < vd; c += 64) { const float v = row[c] * inv; ss += v * v; }
   const float r = 1.0f / sqrtf(wave_sum(ss) / (float)vd + eps);
   for (int c = lane; c < vd; c += 64) {
-    float v = row[c] * inv * r * w[h * vd + c];
+    float v = row[c] * inv * r * w[h * vd + c] * scale;
     if (P) v *= 1.0f / (1.0f + expf(-to_f(P[t * ldp + g0 + h * vd + c])));
     out[item * vd + c] = from_f<T>(v);
   }
 }
 
 extern "C" int ragged_head_norm_gate(const float* o, const float* w, const void* P, int64_t ldp, int g0, void* out, int64_t rows,
-                                     int H, int vd, float eps, int ldo, const float* em, float den_floor, int dtype,
+                                     int H, int vd, float eps, int ldo, const float* em, float den_floor, float scale, int dtype,
                                      hipStream_t st) {
   if (rows <= 0 || H <= 0 || vd <= 0 || rows * H > 0x7fffffff || ldo < vd + (em ? 1 : 0)) return -1;
   const int64_t items = rows * H;
   RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((head_norm_gate_kernel<T>), dim3((unsigned)((items + 3) / 4)), dim3(256), 0, st, o, w,
-                                            (const T*)P, ldp, g0, (T*)out, items, H, vd, eps, ldo, em, den_floor))
+                                            (const T*)P, ldp, g0, (T*)out, items, H, vd, eps, ldo, em, den_floor, scale))
   return RAGGED_LAUNCH_OK();
 }

@@ -618,8 +618,12 @@ extern "C" int ragged_add_norm(float* x, const void* y1, const void* y2, const f
 // ---------------------------------------------------------------------------------------------------------------
 // Activations of a feed-forward's inner channels.  act_cols: out[r, c] = act(P[r, col0 + c]), c < n, with
 // kind 0: gelu through erf, 0.5 z (1 + erf(z / sqrt 2));  1: gelu through tanh, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)));
-// 2: relu(z)^2.  glu_pairs: the inner channels come as neighbouring (gate, up) pairs, out[r, c] = silu(P[r, 2 c]) * P[r, 2 c + 1].
-__device__ __forceinline__ float act_value(float z, int kind) {
+// 2: relu(z)^2;  3: a unit with two curvatures (p0, p1 >= 0 are handed in): p0 z^2 + z / 2 right of zero,
+// (1/2 + p1) (e^z - 1 - z) + z / 2 left of it (both branches and their slopes meet at 0);  4: tanh(z).
+// glu_pairs: the inner channels come as neighbouring (gate, up) pairs, out[r, c] = silu(P[r, 2 c]) * P[r, 2 c + 1].
+__device__ __forceinline__ float act_value(float z, int kind, float p0, float p1) {
+  if (kind == 3) return z > 0.f ? p0 * z * z + 0.5f * z : (0.5f + p1) * (expm1f(z) - z) + 0.5f * z;
+  if (kind == 4) return tanhf(z);
   if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
   if (kind == 1) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
   const float v = fmaxf(z, 0.f);
@@ -630,7 +634,7 @@ __device__ __forceinline__ float act_value(float z, int kind) {
 // 16-byte aligned, n a multiple of the piece), otherwise one element
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void act_cols_kernel(const T* __restrict__ P, int64_t ldp, int col0, T* __restrict__ out, int n,
-                                                       int kind) {
+                                                       int kind, float p0, float p1) {
   constexpr int N = VEC ? 16 / (int)sizeof(T) : 1;
   const int64_t r = blockIdx.y;
   const int c = (blockIdx.x * 256 + threadIdx.x) * N;
@@ -641,10 +645,10 @@ __global__ __launch_bounds__(256) void act_cols_kernel(const T* __restrict__ P, 
     union { uint4 q; T e[N]; } v;
     v.q = *reinterpret_cast<const uint4*>(src);
 #pragma unroll
-    for (int i = 0; i < N; ++i) v.e[i] = from_f<T>(act_value(to_f(v.e[i]), kind));
+    for (int i = 0; i < N; ++i) v.e[i] = from_f<T>(act_value(to_f(v.e[i]), kind, p0, p1));
     *reinterpret_cast<uint4*>(dst) = v.q;
   } else {
-    dst[0] = from_f<T>(act_value(to_f(src[0]), kind));
+    dst[0] = from_f<T>(act_value(to_f(src[0]), kind, p0, p1));
   }
 }
 
@@ -659,9 +663,9 @@ __global__ __launch_bounds__(256) void glu_pairs_kernel(const T* __restrict__ P,
   }
 }
 
-extern "C" int ragged_act_cols(const void* P, int64_t ldp, int col0, void* out, int64_t rows, int n, int kind, int dtype,
-                               hipStream_t st) {
-  if (rows <= 0 || rows > 65535LL * 65535LL || n <= 0 || col0 < 0 || ldp < col0 + n || kind < 0 || kind > 2) return -1;
+extern "C" int ragged_act_cols(const void* P, int64_t ldp, int col0, void* out, int64_t rows, int n, int kind, float p0, float p1,
+                               int dtype, hipStream_t st) {
+  if (rows <= 0 || rows > 65535LL * 65535LL || n <= 0 || col0 < 0 || ldp < col0 + n || kind < 0 || kind > 4) return -1;
   RAGGED_DISPATCH(dtype,
     constexpr int N = 16 / (int)sizeof(T);
     const bool vec = n % N == 0 && ldp % N == 0 && col0 % N == 0 && ((uintptr_t)P % 16) == 0 && ((uintptr_t)out % 16) == 0;
@@ -670,8 +674,9 @@ extern "C" int ragged_act_cols(const void* P, int64_t ldp, int col0, void* out, 
       const unsigned nr = (unsigned)(rows - r0 < 65535 ? rows - r0 : 65535);
       const T* src = (const T*)P + r0 * ldp;
       T* dst = (T*)out + r0 * n;
-      if (vec) hipLaunchKernelGGL((act_cols_kernel<T, true>), dim3((n / N + 255) / 256, nr), dim3(256), 0, st, src, ldp, col0, dst, n, kind);
-      else hipLaunchKernelGGL((act_cols_kernel<T, false>), dim3((n + 255) / 256, nr), dim3(256), 0, st, src, ldp, col0, dst, n, kind);
+      if (vec) hipLaunchKernelGGL((act_cols_kernel<T, true>), dim3((n / N + 255) / 256, nr), dim3(256), 0, st, src, ldp, col0, dst, n, kind,
+                                  p0, p1);
+      else hipLaunchKernelGGL((act_cols_kernel<T, false>), dim3((n + 255) / 256, nr), dim3(256), 0, st, src, ldp, col0, dst, n, kind, p0, p1);
     })
   return RAGGED_LAUNCH_OK();
 }
@@ -681,5 +686,114 @@ extern "C" int ragged_glu_pairs(const void* P, int64_t ldp, void* out, int64_t r
   const int64_t blocks = (rows * n + 255) / 256;
   const unsigned grid = (unsigned)(blocks < 16384 ? blocks : 16384);
   RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((glu_pairs_kernel<T>), dim3(grid), dim3(256), 0, st, (const T*)P, ldp, (T*)out, rows, n))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Pre-norm blocks over a stream that is kept in S copies X[row][s][D] (S = 1: the ordinary residual stream).  One call
+// sits between two sublayers:
+//   y given:    X'[t] = sum_s mix[s][t] X[s] + out[t] * y      for all t from the old copies (prev = [in | out | mix])
+//   nin given:  u = sum_s nin[s] X'[s];  u_out <- u (float);  xa <- w_next * u / sqrt(mean(u^2) + eps)
+// so the write-back of one sublayer, the read-out of the next and its norm pass over a row once.  One workgroup per row.
+// NV > 0: rows of at most 256 NV channels, u stays in registers; NV = 0: any width, u is made again for the second pass.
+constexpr int HC_MAX = 8;
+
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ X, const T* __restrict__ y, const float* __restrict__ prev,
+                                                      const float* __restrict__ nin, const float* __restrict__ w_next,
+                                                      T* __restrict__ xa, float* __restrict__ u_out, int S, int D, float eps) {
+  __shared__ float red[4];
+  __shared__ float cin[HC_MAX], cout[HC_MAX], cmix[HC_MAX * HC_MAX];
+  if (threadIdx.x < S) {
+    cin[threadIdx.x] = nin ? nin[threadIdx.x] : 0.f;
+    cout[threadIdx.x] = y ? prev[S + threadIdx.x] : 0.f;
+  }
+  if (threadIdx.x < S * S) cmix[threadIdx.x] = y ? prev[2 * S + threadIdx.x] : 0.f;
+  __syncthreads();
+  const int64_t row = blockIdx.x;
+  float* xr = X + row * S * D;
+  // the copies of one channel: update from the old values, return what the next sublayer reads
+  auto channel = [&](int c) {
+    float old[HC_MAX], u = 0.f;
+    for (int s = 0; s < S; ++s) old[s] = xr[(int64_t)s * D + c];
+    if (y) {
+      const float yv = to_f(y[row * D + c]);
+      for (int t = 0; t < S; ++t) {
+        float v = cout[t] * yv;
+        for (int s = 0; s < S; ++s) v += cmix[s * S + t] * old[s];
+        xr[(int64_t)t * D + c] = v;
+        u += cin[t] * v;
+      }
+    } else {
+      for (int s = 0; s < S; ++s) u += cin[s] * old[s];
+    }
+    return u;
+  };
+  if (NV > 0) {
+    float uv[NV > 0 ? NV : 1], ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int c = threadIdx.x + 256 * k;
+      uv[k] = c < D ? channel(c) : 0.f;
+      ss += uv[k] * uv[k];
+      if (u_out && c < D) u_out[row * D + c] = uv[k];
+    }
+    if (!xa) return;
+    const float r = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int c = threadIdx.x + 256 * k;
+      if (c < D) xa[row * D + c] = from_f<T>(uv[k] * r * w_next[c]);
+    }
+    return;
+  }
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += 256) {
+    const float u = channel(c);
+    ss += u * u;
+    if (u_out) u_out[row * D + c] = u;
+  }
+  if (!xa) return;
+  const float r = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
+  for (int c = threadIdx.x; c < D; c += 256) {       // (each thread re-reads the copies it has written itself)
+    float u = 0.f;
+    for (int s = 0; s < S; ++s) u += cin[s] * xr[(int64_t)s * D + c];
+    xa[row * D + c] = from_f<T>(u * r * w_next[c]);
+  }
+}
+
+extern "C" int ragged_hc_step(float* X, const void* y, const float* prev, const float* nin, const float* w_next, void* xa,
+                              float* u_out, int64_t rows, int S, int D, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0 || rows > 0x7fffffff || D <= 0 || S <= 0 || S > HC_MAX || !X || (y && !prev) || (xa && (!w_next || !nin)) ||
+      (u_out && !nin)) return -1;
+  RAGGED_DISPATCH(dtype,
+    if (D <= 1024) hipLaunchKernelGGL((hc_step_kernel<T, 4>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin, w_next,
+                                      (T*)xa, u_out, S, D, eps);
+    else if (D <= 4096) hipLaunchKernelGGL((hc_step_kernel<T, 16>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin,
+                                           w_next, (T*)xa, u_out, S, D, eps);
+    else hipLaunchKernelGGL((hc_step_kernel<T, 0>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin, w_next, (T*)xa,
+                            u_out, S, D, eps))
+  return RAGGED_LAUNCH_OK();
+}
+
+// out[r, c] = scale * o[r, c] * sigmoid(P[r, g0 + c]), c < n: a gate per channel on float head outputs, rounded once
+template <typename T>
+__global__ __launch_bounds__(256) void gate_cols_kernel(const float* __restrict__ o, const T* __restrict__ P, int64_t ldp, int g0,
+                                                        T* __restrict__ out, int64_t rows, int n, float scale) {
+  const int64_t total = rows * n;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / n;
+    const int c = (int)(i % n);
+    out[i] = from_f<T>(scale * o[i] * sigmoidf_(to_f(P[r * ldp + g0 + c])));
+  }
+}
+
+extern "C" int ragged_gate_cols(const float* o, const void* P, int64_t ldp, int g0, void* out, int64_t rows, int n, float scale,
+                                int dtype, hipStream_t st) {
+  if (rows <= 0 || n <= 0 || g0 < 0 || ldp < g0 + n) return -1;
+  const int64_t blocks = (rows * n + 255) / 256;
+  const unsigned grid = (unsigned)(blocks < 16384 ? blocks : 16384);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((gate_cols_kernel<T>), dim3(grid), dim3(256), 0, st, o, (const T*)P, ldp, g0, (T*)out, rows,
+                                            n, scale))
   return RAGGED_LAUNCH_OK();
 }

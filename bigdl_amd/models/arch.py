@@ -1235,8 +1235,8 @@ def is_native_arch(config_dict: dict, opt_in: Optional[bool] = None) -> bool:
 # ---------------------------------------------------------------------------------------------
 def ragged_arch(config_dict: dict):
     """The module that builds a ragged engine for this config (``read_config``, ``build_engine``, ``load``), or None."""
-    from . import filanex, lipizen, merusun
-    for mod in (lipizen, merusun, filanex):
+    from . import dimelix, filanex, lipizen, merusun
+    for mod in (lipizen, merusun, filanex, dimelix):
         if config_dict.get("architecture") == mod.ARCHITECTURE:
             return mod
     return None

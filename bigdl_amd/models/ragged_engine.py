@@ -9,9 +9,11 @@ into arbitrary portions next to single decoded tokens run here instead:
   product runs once over all rows; the mixers read ``BatchMeta`` (row -> sequence, position, pages);
 * keys / values live in 64-token pages of a ``PagedStatePool``, per-sequence state in its slots;
 * the mixers are described by small dataclasses whose fields are the design's constants, so a new design is a new list
-  of them (``models/lipizen.py``, ``models/merusun.py`` and ``models/filanex.py`` build one from a ``config.json``);
-* three residual forms: the post-sum norm x <- norm(alpha x + f(x)), the sandwich x <- x + norm_b(f(norm_a(x))), and the
-  parallel pre-norm block u = norm(x), x <- x + mixer(u) + ff(u);
+  of them (``models/lipizen.py``, ``models/merusun.py``, ``models/filanex.py`` and ``models/dimelix.py`` build one from
+  a ``config.json``);
+* four residual forms: the post-sum norm x <- norm(alpha x + f(x)), the sandwich x <- x + norm_b(f(norm_a(x))), the
+  parallel pre-norm block u = norm(x), x <- x + mixer(u) + ff(u), and the sequential pre-norm block x <- x + f(norm(x))
+  per sublayer, whose stream may be kept in several copies that every sublayer reads and rewrites with learned weights;
 * a run of layers may be executed several times with the same weights (every execution has its own cache), with the
   embedding output mixed back into the stream in front of a pass; the embedding may add a row of a token-pair table;
 * matrix products are the library's (bf16 inputs with 32-bit accumulation, or plain float32), everything between them
@@ -62,6 +64,9 @@ class WindowAttention:
     rot_freqs: Optional[tuple] = None  # the pairs' frequencies, if they are not base^(-2 i / rot_dims) / rot_factor
     rot_amp: float = 1.0           # cosine and sine are multiplied by this
     gate_channels: bool = False    # with ``gate``: one sigmoid gate per output channel instead of one per head
+    head_sinks: bool = False       # every head has a learned sink score (``LayerTensors.sinks``) instead of the one number ``sink``
+    dist_slopes: Optional[tuple] = None  # per head: slope * (i - j) is taken off the scaled score of query i and key j
+    v_from_k: bool = False         # no value projection: the values are the key projections as they are before norm and rotation
 
 
 @dataclass
@@ -79,6 +84,32 @@ class LatentAttention:
     rot_dims: int = 0              # leading channels of the rotated part that turn (neighbouring pairs 2 i, 2 i + 1)
     rot_base: float = 10000.0
     window: int = 0
+    gate: bool = False             # one sigmoid gate per output channel, from the mixer's input, behind the value up-projection
+    out_scale: float = 1.0
+
+
+@dataclass
+class DeltaRule:
+    """Generalised delta rule with a matrix state per head (keys, values and receptance of ``dim`` channels each):
+    S <- diag(w) S - (a * n)(n^T S) + k v^T with the unit key n = k / sqrt(|k|^2 + unit_eps), both terms reading the old state;
+    o = S^T r.  The decay w = exp(-decay_rate * sigmoid(W_2 tanh(W_1 h) + b_w)) comes through a low-rank pair of products,
+    the removal rate a = sigmoid(W_a h + b_a); both are per head and key channel.  Each head's output is divided by its
+    root mean square, weighted, gated by a sigmoid of a projection of the mixer's input and multiplied by ``out_scale``."""
+    heads: int
+    dim: int
+    decay_rank: int
+    decay_rate: float = math.exp(-0.5)
+    unit_eps: float = 1e-6
+    out_scale: float = 1.0
+
+
+@dataclass
+class SideBySide:
+    """Two mixers that read the same input; their outputs are summed, each with its own weight (carried by the mixers'
+    ``out_scale``, so that one output projection [W_left | W_right] serves both).  The two must keep different kinds of
+    state (pages against a matrix), since an execution has one cache of each kind."""
+    left: object
+    right: object
 
 
 @dataclass
@@ -134,9 +165,10 @@ class RoutedExperts:
 
 @dataclass
 class DenseMlp:
-    """y = W_down act(W_up h + b_up) + b_down, act "gelu_erf" (0.5 z (1 + erf(z / sqrt 2))), "gelu_tanh" or "relu2".  In the
-    parallel block its up projection is stacked behind the mixer's input projections (one product reads the normed
-    stream once)."""
+    """y = W_down act(W_up h + b_up) + b_down, act "gelu_erf" (0.5 z (1 + erf(z / sqrt 2))), "gelu_tanh", "relu2" or "xielu"
+    (a z^2 + z / 2 right of zero, (1/2 + b)(e^z - 1 - z) + z / 2 left of it, a and b = softplus of two learned numbers of the
+    layer, ``LayerTensors.act_params``).  In the parallel block its up projection is stacked behind the mixer's input
+    projections (one product reads the normed stream once)."""
     ff: int
     act: str = "gelu_erf"
     bias: bool = True
@@ -172,7 +204,9 @@ class RaggedConfig:
     name: str = "ragged"
     embed_scale: float = 1.0
     block: str = "post_sum"        # "post_sum": x <- norm(alpha x + f(x)); "sandwich": x <- x + norm_b(f(norm_a(x)));
-                                   # "parallel": u = norm(x), x <- x + mixer(u) + ff(u)
+                                   # "parallel": u = norm(x), x <- x + mixer(u) + ff(u); "pre_norm": x <- x + f(norm(x)) per sublayer
+    streams: int = 1               # "pre_norm": copies of the stream; every sublayer reads a weighted sum of them and writes
+                                   # X[t] <- sum_s mix[s, t] X[s] + out[t] f(.) (``LayerTensors.hc1 / hc2``); the model's output is their sum
     runs: Optional[list] = None    # layer index of every layer execution, in order (None: every layer once); an execution
                                    # has its own cache / state, whatever weights it shares
     mix_in: tuple = ()             # executions in front of which x <- W_mix [x ; embedding output]
@@ -209,6 +243,17 @@ class LayerTensors:
     w_sup: Optional[torch.Tensor] = None     # shared expert
     w_sdn: Optional[torch.Tensor] = None
     b_down: Optional[torch.Tensor] = None    # dense feed-forward: bias of the down projection (the up bias is part of b_in)
+    w_ff: Optional[torch.Tensor] = None      # dense feed-forward of the sequential pre-norm block: its up projection
+    act_params: Optional[tuple] = None       # the two curvatures of an "xielu" feed-forward (floats, softplus already applied)
+    sinks: Optional[torch.Tensor] = None     # float [heads]: learned sink scores
+    slopes: Optional[torch.Tensor] = None    # float [heads]: distance slopes
+    hc1: Optional[torch.Tensor] = None       # float [2 S + S S]: read-out, write-back and mixing weights of the stream copies
+    hc2: Optional[torch.Tensor] = None       # around the mixer (hc1) and the feed-forward (hc2)
+    w_decay: Optional[torch.Tensor] = None   # delta rule: second product of the decay's low-rank pair [heads dim, rank]
+    decay_bias: Optional[torch.Tensor] = None  # float [heads dim]
+    remove_bias: Optional[torch.Tensor] = None  # float [heads dim]
+    left: Optional["LayerTensors"] = None    # side-by-side mixers: what each of the two needs beyond the shared projections
+    right: Optional["LayerTensors"] = None
 
 
 def rotary_inv_freq(dims: int, base: float, factor: float) -> torch.Tensor:
@@ -269,6 +314,18 @@ class RaggedDecoder:
                                      "the same head layout")
                 self._kv_run[ri] = latest[m.kv_from]
             latest[li] = ri
+        if cfg.block == "pre_norm":
+            S = cfg.streams
+            if not 1 <= S <= 8:
+                raise ValueError("1 to 8 copies of the stream")
+            # read-out weights that sum the copies (the model's output), and the coefficients of a plain residual sum
+            self._sum_read = torch.cat([torch.ones(2 * S), torch.eye(S).reshape(-1)]).to(self.device)
+            for lt in layers:
+                for name in ("hc1", "hc2"):
+                    if getattr(lt, name) is None:
+                        if S != 1:
+                            raise ValueError("several copies of the stream need every sublayer's coefficients")
+                        setattr(lt, name, self._sum_read)
         self.first_cost = self.rest_cost_mean = self.peak_memory = 0.0
         # BIGDL_RAGGED_GRAPH=1: steps that carry one token per sequence are recorded once per (sequences, page-table
         # width) and replayed as one hipGraph.  Off by default: every step is issued kernel by kernel.  With recording
@@ -282,28 +339,39 @@ class RaggedDecoder:
         """what every layer execution keeps, by execution index"""
         specs = {}
         for ri, li in enumerate(self.runs):
-            m = self.cfg.mixers[li]
+            top = self.cfg.mixers[li]
             s = []
-            if isinstance(m, WindowAttention):
-                if m.kv_from is None:
-                    s.append(("kv", m.kv_heads, m.maps * m.dim, m.vdim))
-                if m.conv_taps > 1:
-                    s.append(("tail", m.conv_taps - 1, self._conv_channels(m)))
-            elif isinstance(m, LatentAttention):
-                s.append(("k", 1, m.rank + m.rot_dim))          # values are the rows' leading channels
-            elif isinstance(m, Hgrn2):
-                s.append(("matrix", m.heads, m.dim, m.vdim))
-            elif isinstance(m, Mlstm):
-                s.append(("matrix", m.heads, m.dim, m.vdim + 1))  # S and, as its last column, the normaliser n
-                s.append(("vector", m.heads))                   # the running maximum of every head
+            for m in ((top.left, top.right) if isinstance(top, SideBySide) else (top,)):
+                s += self._mixer_specs(m)
+            kinds = [spec[0] if spec[0] != "kv" else "k" for spec in s]
+            if len(set(kinds)) != len(kinds):
+                raise ValueError(f"layer {li}: mixers side by side must keep different kinds of state")
             specs[ri] = s
         return specs
+
+    def _mixer_specs(self, m):
+        s = []
+        if isinstance(m, WindowAttention):
+            if m.kv_from is None:
+                s.append(("kv", m.kv_heads, m.maps * m.dim, m.vdim))
+            if m.conv_taps > 1:
+                s.append(("tail", m.conv_taps - 1, self._conv_channels(m)))
+        elif isinstance(m, LatentAttention):
+            s.append(("k", 1, m.rank + m.rot_dim))          # values are the rows' leading channels
+        elif isinstance(m, Hgrn2):
+            s.append(("matrix", m.heads, m.dim, m.vdim))
+        elif isinstance(m, Mlstm):
+            s.append(("matrix", m.heads, m.dim, m.vdim + 1))  # S and, as its last column, the normaliser n
+            s.append(("vector", m.heads))                   # the running maximum of every head
+        elif isinstance(m, DeltaRule):
+            s.append(("matrix", m.heads, m.dim, m.dim))
+        return s
 
     @staticmethod
     def _conv_channels(m: WindowAttention) -> int:
         c = m.heads * m.maps * m.dim
         if m.kv_from is None:
-            c += m.kv_heads * (m.maps * m.dim + m.vdim)
+            c += m.kv_heads * (m.maps * m.dim + (0 if m.v_from_k else m.vdim))
         return c
 
     def ensure_pool(self, max_tokens: int, slots: int) -> PagedStatePool:
@@ -329,16 +397,19 @@ class RaggedDecoder:
         if m.kv_from is None:
             ops.conv_head(P, cq, meta, ch0=cq, ngroups=m.kv_heads * m.maps, gsize=m.dim, normw=lt.k_norm, eps=eps,
                           rot=m.rot_dims, inv_freq=lt.inv_freq, pages=pool.k[li], **conv, **turn)
-            ops.conv_head(P, cq + ck, meta, ch0=cq + ck, ngroups=m.kv_heads, gsize=m.vdim, normw=None, eps=eps, rot=0,
+            # values: their own projection, or the key projections once more as they came (no norm, no rotation)
+            cv = cq if m.v_from_k else cq + ck
+            ops.conv_head(P, cv, meta, ch0=cv, ngroups=m.kv_heads, gsize=m.vdim, normw=None, eps=eps, rot=0,
                           inv_freq=None, pages=pool.v[li], **conv)
-            col = cq + ck + m.kv_heads * m.vdim
+            col = cq + ck + (0 if m.v_from_k else m.kv_heads * m.vdim)
         if m.conv_taps > 1:
             ops.conv_state(P, 0, pool.tail[li], m.conv_taps, conv["C"], meta)
         src = self._kv_run[li]
         return ops.paged_attn(q, pool.k[src], pool.v[src], meta, maps=m.maps, H=m.heads, G=m.kv_heads, d=m.dim, vd=m.vdim,
                               window=m.window, keep_first=m.keep_first, scale=m.scale, lam=m.lam, out_scale=m.out_scale,
                               out_norm=m.out_norm, eps=eps, gate=P if m.gate else None, gate0=col, sink=m.sink,
-                              chunk=m.chunk, softcap=m.softcap, gate_wide=m.gate and m.gate_channels)
+                              chunk=m.chunk, softcap=m.softcap, gate_wide=m.gate and m.gate_channels,
+                              sinks=lt.sinks if m.head_sinks else None, slopes=lt.slopes if m.dist_slopes is not None else None)
 
     def _latent(self, li, m: LatentAttention, lt: LayerTensors, P, meta):
         """Scores of head h are q_h . [W_uk,h c | rotated part] = [W_uk,h^T q_h | rotated query part] . [c | rotated part]:
@@ -358,7 +429,32 @@ class RaggedDecoder:
         q[:, :, m.rank:] = q3[:, :, m.dim:]
         o = ops.paged_attn(q.view(T, -1), pool.k[li], pool.k[li], meta, maps=1, H=H, G=1, d=m.rank + m.rot_dim, vd=m.rank,
                            window=m.window, keep_first=0, scale=m.scale, lam=0.0, out_scale=1.0, out_norm=False, eps=eps)
-        return torch.bmm(o.view(T, H, m.rank).transpose(0, 1), lt.w_uv.transpose(1, 2)).transpose(0, 1).reshape(T, H * m.vdim)
+        o = o.view(T, H, m.rank).transpose(0, 1)
+        if not m.gate and m.out_scale == 1.0:
+            return torch.bmm(o, lt.w_uv.transpose(1, 2)).transpose(0, 1).reshape(T, H * m.vdim)
+        # gated: the head outputs stay float up to the gate, which rounds them once
+        if o.dtype == torch.float32 or o.device.type != "cuda":
+            of = torch.bmm(o.float(), lt.w_uv.float().transpose(1, 2))
+        else:
+            of = torch.bmm(o, lt.w_uv.transpose(1, 2), out_dtype=torch.float32)
+        of = of.transpose(0, 1).reshape(T, H * m.vdim)
+        if not m.gate:
+            return (of * m.out_scale).to(self.act)
+        return ops.gate_cols(of, P, H * hd + m.rank + m.rot_dim, self.act, m.out_scale)
+
+    def _delta(self, li, m: DeltaRule, lt: LayerTensors, P, meta):
+        ops = self.ops
+        hd = m.heads * m.dim
+        # columns of P: r | k | v | output gate | removal logits | low-rank decay input
+        lo = ops.act_cols(P, 5 * hd, m.decay_rank, "tanh")
+        arrays = ops.delta_gates(P, 0, hd, 4 * hd, self._linear_f32(lo, lt.w_decay), lt.decay_bias, lt.remove_bias, m.decay_rate,
+                                 m.unit_eps, m.heads, m.dim)
+        o = ops.delta_scan(arrays, P, 2 * hd, self.pool.matrix[li], m.heads, m.dim, m.dim, meta)
+        return ops.head_norm_gate(o, lt.o_norm, P, 3 * hd, m.heads, m.dim, self.cfg.norm_eps, self.act, scale=m.out_scale)
+
+    def _side_by_side(self, li, m: SideBySide, lt: LayerTensors, P, meta):
+        nl = lt.left.w_in.shape[0]                   # the left mixer's rows of the stacked projection
+        return torch.cat([self._mixer(li, m.left, lt.left, P[:, :nl], meta), self._mixer(li, m.right, lt.right, P[:, nl:], meta)], 1)
 
     def _mlstm(self, li, m: Mlstm, lt: LayerTensors, P, meta):
         ops, pool = self.ops, self.pool
@@ -492,6 +588,10 @@ class RaggedDecoder:
             return self._latent(li, m, lt, P, meta)
         if isinstance(m, Mlstm):
             return self._mlstm(li, m, lt, P, meta)
+        if isinstance(m, DeltaRule):
+            return self._delta(li, m, lt, P, meta)
+        if isinstance(m, SideBySide):
+            return self._side_by_side(li, m, lt, P, meta)
         return self._hgrn2(li, m, lt, P, meta)
 
     def _forward(self, meta, idt, rows, collect):
@@ -504,6 +604,8 @@ class RaggedDecoder:
             self._sandwich_layers(x, meta, collect)
         elif cfg.block == "parallel":
             x = self._parallel_layers(x, meta, collect)
+        elif cfg.block == "pre_norm":
+            x = self._prenorm_layers(x, meta, collect)
         else:
             xa = x.to(self.act)
             for ri, li in enumerate(self.runs):
@@ -578,6 +680,33 @@ class RaggedDecoder:
             if collect is not None:
                 collect.append(x.clone())
         return x
+
+    def _prenorm_layers(self, x, meta, collect):
+        """x <- x + f(norm(x)) for the mixer and then the feed-forward of every execution, on a stream of ``cfg.streams``
+        copies X[s] (all equal to the embedding output at first): sublayer f reads u = sum_s in[s] X[s] and writes
+        X[t] <- sum_s mix[s, t] X[s] + out[t] f(norm(u)).  The write-back of one sublayer, the read-out of the next and its
+        norm are one kernel.  Returns the sum of the copies."""
+        cfg, ops, eps = self.cfg, self.ops, self.cfg.norm_eps
+        S = cfg.streams
+        X = x[:, None, :].repeat(1, S, 1)
+        y = prev = None
+        for ri, li in enumerate(self.runs):
+            m, mlp, lt = cfg.mixers[li], cfg.mlps[li], self.layers[li]
+            xa, _ = ops.hc_step(X, y, prev, lt.hc1, lt.norm1, eps, self.act)
+            y, prev = F.linear(self._mixer(ri, m, lt, F.linear(xa, lt.w_in, lt.b_in), meta), lt.w_out), lt.hc1
+            if isinstance(mlp, DenseMlp):
+                if mlp.bias:
+                    raise ValueError("the sequential pre-norm block's dense feed-forward has no biases")
+                xa, _ = ops.hc_step(X, y, prev, lt.hc2, lt.norm2, eps, self.act)
+                a = F.linear(xa, lt.w_ff)
+                y, prev = F.linear(ops.act_cols(a, 0, mlp.ff, mlp.act, lt.act_params or (0.0, 0.0)), lt.w_down, lt.b_down), lt.hc2
+            elif mlp is not None:
+                raise ValueError("the sequential pre-norm block has no such feed-forward yet")
+            if collect is not None:
+                ops.hc_step(X, y, prev, None, None, eps, self.act)
+                y = prev = None
+                collect.append(X.sum(1))
+        return ops.hc_step(X, y, prev, self._sum_read, None, eps, self.act, want_u=True)[1]
 
     def _linear_f32(self, a, w):
         """a w^T with the operands in the activation type and a float32 result (no rounding of the 32-bit accumulator)"""

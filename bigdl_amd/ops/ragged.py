@@ -92,7 +92,8 @@ class _AttnArgs(ctypes.Structure):
                 ("out_scale", ctypes.c_float), ("out_norm", ctypes.c_int), ("eps", ctypes.c_float),
                 ("rows", ctypes.c_void_p), ("n_rows", ctypes.c_int), ("tiles", ctypes.c_void_p), ("n_tiles", ctypes.c_int),
                 ("ldv", ctypes.c_int64), ("sink", ctypes.c_int), ("sink_score", ctypes.c_float), ("chunk", ctypes.c_int),
-                ("softcap", ctypes.c_float), ("gate_wide", ctypes.c_int)]
+                ("softcap", ctypes.c_float), ("gate_wide", ctypes.c_int), ("sinks", ctypes.c_void_p),
+                ("slopes", ctypes.c_void_p)]
 
 
 def lib():
@@ -111,11 +112,15 @@ def lib():
         L.ragged_post_norm_add.argtypes = [vp, vp, vp, vp, vp, i64, ci, cf, ci, vp]
         L.ragged_mlstm_gates.argtypes = [vp, i64, ci, vp, cf, cf, vp, vp, vp, vp, ci, _Batch, ci, vp]
         L.ragged_mlstm_expand.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
-        L.ragged_head_norm_gate.argtypes = [vp, vp, vp, i64, ci, vp, i64, ci, ci, cf, ci, vp, cf, ci, vp]
+        L.ragged_head_norm_gate.argtypes = [vp, vp, vp, i64, ci, vp, i64, ci, ci, cf, ci, vp, cf, cf, ci, vp]
         L.ragged_moe_route.argtypes = [vp, i64, vp, vp, vp, i64, ci, ci, ci, ci, ci, cf, ci, ci, ci, ci, vp]
         L.ragged_embed_rows.argtypes = [vp, vp, vp, vp, cf, vp, i64, ci, ci, vp]
         L.ragged_add_norm.argtypes = [vp, vp, vp, vp, vp, i64, ci, cf, ci, vp]
-        L.ragged_act_cols.argtypes = [vp, i64, ci, vp, i64, ci, ci, ci, vp]
+        L.ragged_act_cols.argtypes = [vp, i64, ci, vp, i64, ci, ci, cf, cf, ci, vp]
+        L.ragged_hc_step.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, cf, ci, vp]
+        L.ragged_gate_cols.argtypes = [vp, vp, i64, ci, vp, i64, ci, cf, ci, vp]
+        L.ragged_delta_gates.argtypes = [vp, i64, ci, ci, ci, vp, vp, vp, cf, cf, vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
+        L.ragged_delta_scan.argtypes = [vp, vp, vp, vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, ci, _Batch, ci, vp]
         L.ragged_glu_pairs.argtypes = [vp, i64, vp, i64, ci, ci, vp]
         L.ragged_relu2.argtypes = [vp, vp, i64, ci, vp]
         L.ragged_moe_combine.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
@@ -435,11 +440,15 @@ class HipOps:
         return out
 
     def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
-                   eps, gate=None, gate0=0, sink=None, chunk=0, softcap=0.0, gate_wide=False):
+                   eps, gate=None, gate0=0, sink=None, chunk=0, softcap=0.0, gate_wide=False, sinks=None, slopes=None):
         """``vpages`` may be ``kpages`` itself: the values are then the leading ``vd`` channels of the key rows.
         ``chunk`` > 0: a key is visible only inside the query's block of that many positions; ``softcap`` > 0: scores go
-        through softcap * tanh(. / softcap); ``gate_wide``: one gate column per output channel instead of one per head."""
-        _f32(q)
+        through softcap * tanh(. / softcap); ``gate_wide``: one gate column per output channel instead of one per head;
+        ``sinks`` float [H]: every head's own sink score (instead of the one number ``sink``); ``slopes`` float [H]:
+        slopes[h] * (i - j) is taken off the scaled score of query i and key j."""
+        _f32(q, sinks, slopes)
+        if any(t is not None and t.numel() != H for t in (sinks, slopes)):
+            raise ValueError("one sink score / one slope per query head")
         _act(kpages, vpages, gate)
         _page_check(meta, kpages)
         _page_check(meta, vpages)
@@ -463,9 +472,13 @@ class HipOps:
         a.ldv = vpages.shape[3]
         if sink is not None:
             a.sink, a.sink_score = 1, float(sink)
+        if sinks is not None:
+            a.sink, a.sinks = 1, sinks.data_ptr()
+        if slopes is not None:
+            a.slopes = slopes.data_ptr()
         if kpages.dtype == torch.bfloat16 and self.mfma and maps == 1 and not lib().ragged_paged_attn_mfma_ok(d, vd) \
                 and lib().ragged_paged_attn_mfma_wide_ok(d, vd) and a.ldv % 8 == 0 and not keep_first and not out_norm \
-                and gate is None and not chunk and not softcap:
+                and gate is None and not chunk and not softcap and sinks is None and slopes is None:
             # rows too wide for the row-wise kernel's lanes: long portions as tiles of 64 rows of one head, single tokens
             # and short portions with 16 heads of a row side by side, both on the matrix cores
             tiles, n_tiles, rows, n_rows = meta.attn_split(self.mfma_min_rows)
@@ -512,9 +525,10 @@ class HipOps:
             _ok(lib().ragged_relu2(A.data_ptr(), out.data_ptr(), A.numel(), _DT[A.dtype], _stream()), "relu2")
         return out
 
-    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act, em=None, den_floor=0.0):
-        """each head's rows of ``o`` divided by their root mean square, times ``w``, times sigmoid(gate columns of P).  With
-        ``em`` [T, H]: ``o`` has vd + 1 columns per head and is first divided by max(|last column|, em) + den_floor."""
+    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act, em=None, den_floor=0.0, scale=1.0):
+        """each head's rows of ``o`` divided by their root mean square, times ``w``, times sigmoid(gate columns of P), times
+        ``scale``.  With ``em`` [T, H]: ``o`` has vd + 1 columns per head and is first divided by max(|last column|, em) +
+        den_floor."""
         _f32(o, w, em)
         _act(P)
         T = o.shape[0]
@@ -524,8 +538,8 @@ class HipOps:
             raise ValueError("head outputs / gate columns do not fit")
         out = torch.empty(T, H * vd, dtype=act, device=o.device)
         _ok(lib().ragged_head_norm_gate(o.data_ptr(), w.data_ptr(), P.data_ptr(), P.stride(0), g0, out.data_ptr(), T, H, vd, eps,
-                                        ldo, None if em is None else em.data_ptr(), den_floor, _DT[act], _stream()),
-            "head_norm_gate")
+                                        ldo, None if em is None else em.data_ptr(), den_floor, float(scale), _DT[act],
+                                        _stream()), "head_norm_gate")
         return out
 
     def mlstm_gates(self, P, i0, gate_bias, cap, m_start, H, mstate, meta):
@@ -673,16 +687,17 @@ class HipOps:
                                   _DT[act], _stream()), "add_norm")
         return xa
 
-    _ACT_KINDS = {"gelu_erf": 0, "gelu_tanh": 1, "relu2": 2}
+    _ACT_KINDS = {"gelu_erf": 0, "gelu_tanh": 1, "relu2": 2, "xielu": 3, "tanh": 4}
 
-    def act_cols(self, P, col0, n, kind):
-        """act(P[:, col0 : col0 + n]) as a contiguous [rows, n] matrix; kind: gelu_erf, gelu_tanh or relu2."""
+    def act_cols(self, P, col0, n, kind, params=(0.0, 0.0)):
+        """act(P[:, col0 : col0 + n]) as a contiguous [rows, n] matrix; kind: gelu_erf, gelu_tanh, relu2, tanh, or xielu with
+        ``params`` = (a, b) >= 0: a z^2 + z / 2 right of zero, (1/2 + b)(e^z - 1 - z) + z / 2 left of it."""
         _act(P)
         if P.dim() != 2 or col0 < 0 or col0 + n > P.shape[1]:
             raise ValueError("columns outside the matrix")
         out = torch.empty(P.shape[0], n, dtype=P.dtype, device=P.device)
-        _ok(lib().ragged_act_cols(P.data_ptr(), P.stride(0), col0, out.data_ptr(), P.shape[0], n, self._ACT_KINDS[kind], _DT[P.dtype],
-                                  _stream()), "act_cols")
+        _ok(lib().ragged_act_cols(P.data_ptr(), P.stride(0), col0, out.data_ptr(), P.shape[0], n, self._ACT_KINDS[kind], float(params[0]),
+                                  float(params[1]), _DT[P.dtype], _stream()), "act_cols")
         return out
 
     def glu_pairs(self, P):
@@ -694,6 +709,104 @@ class HipOps:
         if out.numel():
             _ok(lib().ragged_glu_pairs(P.data_ptr(), P.stride(0), out.data_ptr(), P.shape[0], P.shape[1] // 2, _DT[P.dtype], _stream()),
                 "glu_pairs")
+        return out
+
+
+    def hc_step(self, X, y, prev, nxt, w_next, eps, act, want_u=False):
+        """The stream in S copies, X float [rows, S, D], between two sublayers.  ``prev`` / ``nxt``: float [2 S + S S] =
+        [read-out weights | write-back weights | mixing matrix (from, to)] of the sublayer that produced ``y`` and of the
+        one that reads next.  With ``y``: X[t] <- sum_s mix[s, t] X[s] + out[t] y in place.  With ``nxt``: u = sum_s in[s] X[s];
+        returns (w_next * rmsnorm(u) as ``act`` or None, u as float if ``want_u`` else None)."""
+        _f32(X, prev, nxt, w_next)
+        _act(y)
+        rows, S, D = X.shape
+        if S > 8 or (y is not None and (prev is None or y.shape != (rows, D) or not y.is_contiguous() or y.dtype != act)) \
+                or any(c is not None and c.numel() != 2 * S + S * S for c in (prev, nxt)) \
+                or (w_next is not None and (nxt is None or w_next.numel() != D)) or (want_u and nxt is None):
+            raise ValueError("stream copies / coefficients / sublayer output do not fit")
+        xa = None if w_next is None else torch.empty(rows, D, dtype=act, device=X.device)
+        u = torch.empty(rows, D, dtype=torch.float32, device=X.device) if want_u else None
+        _ok(lib().ragged_hc_step(X.data_ptr(), None if y is None else y.data_ptr(), None if prev is None else prev.data_ptr(),
+                                 None if nxt is None else nxt.data_ptr(), None if w_next is None else w_next.data_ptr(),
+                                 None if xa is None else xa.data_ptr(), None if u is None else u.data_ptr(), rows, S, D, eps,
+                                 _DT[act], _stream()), "hc_step")
+        return xa, u
+
+    def gate_cols(self, o, P, g0, act, scale=1.0):
+        """scale * o * sigmoid(P[:, g0 : g0 + n]) for float head outputs o [rows, n], rounded once to ``act``"""
+        _f32(o)
+        _act(P)
+        rows, n = o.shape
+        if P.shape[0] != rows or g0 < 0 or g0 + n > P.shape[1] or P.dtype != act:
+            raise ValueError("gate columns outside the projection matrix")
+        out = torch.empty(rows, n, dtype=act, device=o.device)
+        _ok(lib().ragged_gate_cols(o.data_ptr(), P.data_ptr(), P.stride(0), g0, out.data_ptr(), rows, n, float(scale), _DT[act],
+                                   _stream()), "gate_cols")
+        return out
+
+    def delta_gates(self, P, r0, k0, a0, wl, w0, ab, rate, tiny, H, d):
+        """The delta-rule scan's arrays, float [T, H d] each: r, decay exp(-rate sigmoid(wl + w0)), unit key n = k / sqrt(|k|^2
+        + tiny) per head, removal sigmoid(a + ab) * n, and k.  r, k and the removal logits are columns of P; ``wl`` [T, H d]
+        float are the decay logits."""
+        _act(P)
+        _f32(wl, w0, ab)
+        T, HD = P.shape[0], H * d
+        if max(r0, k0, a0) + HD > P.shape[1] or wl.shape != (T, HD) or w0.numel() != HD or ab.numel() != HD:
+            raise ValueError("delta-rule columns / biases do not fit")
+        outs = [torch.empty(T, HD, dtype=torch.float32, device=P.device) for _ in range(5)]
+        _ok(lib().ragged_delta_gates(P.data_ptr(), P.stride(0), r0, k0, a0, wl.data_ptr(), w0.data_ptr(), ab.data_ptr(), float(rate),
+                                     float(tiny), *[t.data_ptr() for t in outs], T, H, d, _DT[P.dtype], _stream()), "delta_gates")
+        return outs
+
+    delta_chunk = 64          # portions of at least four times this many tokens run the delta rule in chunks
+
+    def delta_scan(self, arrays, P, v0, state, H, d, vd, meta):
+        """S <- diag(w) S - b (n^T S) + k v^T, o = S^T r per head over this step's rows; ``arrays`` = (r, w, n, b, k) from
+        ``delta_gates``, v = columns v0 .. of P, ``state`` float [slots, H, d, vd].  Returns o float [T, H vd]."""
+        _f32(state, *arrays)
+        _act(P)
+        if any(a.shape != (meta.T, H * d) for a in arrays) or v0 + H * vd > P.shape[1] or P.shape[0] != meta.T \
+                or state.shape[1:] != (H, d, vd) or max(s[0] for s in meta.seqs) >= state.shape[0]:
+            raise ValueError("recurrent state / scan arrays do not fit")
+        out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
+        L, dt, st = lib(), _DT[P.dtype], _stream()
+        ptrs = [a.data_ptr() for a in arrays]
+        longest = max(n for _, _, n, _ in meta.seqs)
+        if longest < 4 * self.delta_chunk:
+            _ok(L.ragged_delta_scan(*ptrs, P.data_ptr(), P.stride(0), v0, state.data_ptr(), out.data_ptr(), H, d, vd, 1, meta.c(),
+                                    dt, st), "delta_scan")
+            return out
+        # Long portions: chunks side by side.  A chunk maps its start state linearly, S_end = A S_start + L: L is the chunk
+        # scanned from zero, A (d x d per head) the chunk scanned without inputs from the identity.  The chunk-start states
+        # follow one after the other from those, and the chunks are scanned again from them for the outputs.
+        nc, cstart, zeros, ones, cid, cfirst, last = meta.chunks(self.delta_chunk)
+        local = torch.empty(nc, H, d, vd, dtype=torch.float32, device=P.device)
+        trans = torch.eye(d, dtype=torch.float32, device=P.device).repeat(nc, H, 1, 1)
+
+        def chunk_batch(past):
+            return _Batch(None, None, cstart.data_ptr(), past.data_ptr(), cid.data_ptr(), None, meta.T, nc, 0)
+        _ok(L.ragged_delta_scan(*ptrs, P.data_ptr(), P.stride(0), v0, local.data_ptr(), None, H, d, vd, 1, chunk_batch(zeros), dt, st),
+            "delta_scan (chunks from zero)")
+        _ok(L.ragged_delta_scan(*ptrs, None, 0, 0, trans.data_ptr(), None, H, d, d, 0, chunk_batch(ones), dt, st),
+            "delta_scan (transition matrices)")
+        begin = torch.empty_like(local)
+        first, count = {}, {}
+        at = 0
+        for b, (slot, past, n, _) in enumerate(meta.seqs):
+            first[b], count[b] = at, -(-n // self.delta_chunk)
+            at += count[b]
+        slots = torch.tensor([s[0] for s in meta.seqs], dtype=torch.int64, device=P.device)
+        fresh = torch.tensor([s[1] == 0 for s in meta.seqs], device=P.device)
+        S = torch.where(fresh[:, None, None, None], torch.zeros((), device=P.device), state[slots])      # [B, H, d, vd]
+        for j in range(max(count.values())):                 # the j-th chunk of every sequence that has one
+            bs = [b for b in range(meta.B) if count[b] > j]
+            cs = torch.tensor([first[b] + j for b in bs], dtype=torch.int64, device=P.device)
+            bi = torch.tensor(bs, dtype=torch.int64, device=P.device)
+            begin[cs] = S[bi]
+            S[bi] = torch.matmul(trans[cs], S[bi]) + local[cs]
+        _ok(L.ragged_delta_scan(*ptrs, P.data_ptr(), P.stride(0), v0, begin.data_ptr(), out.data_ptr(), H, d, vd, 1,
+                                chunk_batch(ones), dt, st), "delta_scan (chunks from their start states)")
+        state[slots] = S
         return out
 
 
@@ -800,7 +913,7 @@ class TorchOps:
         return (v if w is None else v * w).to(act)
 
     def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
-                   eps, gate=None, gate0=0, sink=None, chunk=0, softcap=0.0, gate_wide=False):
+                   eps, gate=None, gate0=0, sink=None, chunk=0, softcap=0.0, gate_wide=False, sinks=None, slopes=None):
         out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=q.device)
         q = q.view(meta.T, H, maps, d)
         for b, (slot, past, n, pg) in enumerate(meta.seqs):
@@ -820,15 +933,18 @@ class TorchOps:
             o = None
             for mp in range(maps):
                 s = torch.einsum("thd,hld->htl", qs[:, :, mp], k[:, :, mp].repeat_interleave(rep, 0)) * scale
+                if slopes is not None:
+                    s = s - slopes.view(H, 1, 1) * (i - j).float()
                 if softcap > 0:
                     s = softcap * torch.tanh(s / softcap)
                 s = s.masked_fill(~vis, float("-inf"))
-                if sink is None:
+                if sink is None and sinks is None:
                     w = torch.softmax(s, -1)
                 else:                                     # one more score in the normaliser, no value behind it
-                    top = s.max(-1, keepdim=True).values.clamp(min=sink)
+                    sk = sinks.view(H, 1, 1) if sinks is not None else torch.full((H, 1, 1), float(sink))
+                    top = torch.maximum(s.max(-1, keepdim=True).values, sk)
                     w = torch.exp(s - top)
-                    w = w / (w.sum(-1, keepdim=True) + torch.exp(sink - top))
+                    w = w / (w.sum(-1, keepdim=True) + torch.exp(sk - top))
                 a = w @ v.repeat_interleave(rep, 0)       # [H, n, vd]
                 o = a if mp == 0 else o - lam * a
             o = o.permute(1, 0, 2)
@@ -851,12 +967,12 @@ class TorchOps:
     def relu2(self, A):
         return torch.relu(A.float()).pow(2).to(A.dtype)
 
-    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act, em=None, den_floor=0.0):
+    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act, em=None, den_floor=0.0, scale=1.0):
         v = o.view(o.shape[0], H, -1)
         if em is not None:
             v = v[..., :vd] / (torch.maximum(v[..., vd].abs(), em) + den_floor)[..., None]
         v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(-1, H * vd)
-        return (v * w * torch.sigmoid(P[:, g0:g0 + H * vd].float())).to(act)
+        return (v * w * scale * torch.sigmoid(P[:, g0:g0 + H * vd].float())).to(act)
 
     def mlstm_gates(self, P, i0, gate_bias, cap, m_start, H, mstate, meta):
         li = cap * torch.tanh((P[:, i0:i0 + H].float() + gate_bias[:H]) / cap)
@@ -921,18 +1037,57 @@ class TorchOps:
             return None
         return (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w_next).to(act)
 
-    def act_cols(self, P, col0, n, kind):
+    def act_cols(self, P, col0, n, kind, params=(0.0, 0.0)):
         z = P[:, col0:col0 + n].float()
         if kind == "gelu_erf":
             v = 0.5 * z * (1.0 + torch.erf(z * 0.7071067811865476))
         elif kind == "gelu_tanh":
             v = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        elif kind == "tanh":
+            v = torch.tanh(z)
+        elif kind == "xielu":
+            v = torch.where(z > 0, params[0] * z * z + 0.5 * z, (0.5 + params[1]) * (torch.expm1(z.clamp(max=0.0)) - z) + 0.5 * z)
         else:
             v = torch.relu(z).pow(2)
         return v.to(P.dtype)
 
     def glu_pairs(self, P):
         return (F.silu(P[:, 0::2].float()) * P[:, 1::2].float()).to(P.dtype)
+
+    def hc_step(self, X, y, prev, nxt, w_next, eps, act, want_u=False):
+        S = X.shape[1]
+        if y is not None:
+            out, mix = prev[S:2 * S], prev[2 * S:].view(S, S)
+            X.copy_(torch.einsum("st,rsd->rtd", mix, X) + out[None, :, None] * y.float()[:, None, :])
+        if nxt is None:
+            return None, None
+        u = torch.einsum("s,rsd->rd", nxt[:S], X)
+        xa = None if w_next is None else (u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w_next).to(act)
+        return xa, (u if want_u else None)
+
+    def gate_cols(self, o, P, g0, act, scale=1.0):
+        return (scale * o * torch.sigmoid(P[:, g0:g0 + o.shape[1]].float())).to(act)
+
+    def delta_gates(self, P, r0, k0, a0, wl, w0, ab, rate, tiny, H, d):
+        T, HD = P.shape[0], H * d
+        k = P[:, k0:k0 + HD].float()
+        n = (k.view(T, H, d) / torch.sqrt(k.view(T, H, d).pow(2).sum(-1, keepdim=True) + tiny)).reshape(T, HD)
+        return [P[:, r0:r0 + HD].float(), torch.exp(-rate * torch.sigmoid(wl + w0)), n,
+                torch.sigmoid(P[:, a0:a0 + HD].float() + ab) * n, k]
+
+    def delta_scan(self, arrays, P, v0, state, H, d, vd, meta):
+        rf, wf, nf, bf, kf = arrays
+        out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
+        for b, (slot, past, n, _) in enumerate(meta.seqs):
+            S = state[slot].clone() if past > 0 else torch.zeros_like(state[slot])
+            for i in range(n):
+                t = meta.start[b] + i
+                v = P[t, v0:v0 + H * vd].float().view(H, 1, vd)
+                dot = (nf[t].view(H, d, 1) * S).sum(1, keepdim=True)
+                S = wf[t].view(H, d, 1) * S - bf[t].view(H, d, 1) * dot + kf[t].view(H, d, 1) * v
+                out[t] = (S * rf[t].view(H, d, 1)).sum(1).reshape(-1)
+            state[slot] = S
+        return out
 
 
 def ops_for(device) -> object:
