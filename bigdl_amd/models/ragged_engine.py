@@ -320,8 +320,8 @@ class RaggedDecoder:
                 raise ValueError("1 to 8 copies of the stream")
             # read-out weights that sum the copies (the model's output), and the coefficients of a plain residual sum
             self._sum_read = torch.cat([torch.ones(2 * S), torch.eye(S).reshape(-1)]).to(self.device)
-            for lt in layers:
-                for name in ("hc1", "hc2"):
+            for lt, mlp in zip(layers, cfg.mlps):
+                for name in ("hc1", "hc2") if mlp is not None else ("hc1",):
                     if getattr(lt, name) is None:
                         if S != 1:
                             raise ValueError("several copies of the stream need every sublayer's coefficients")
