@@ -3,7 +3,7 @@ the reference's all-in-one protocol (python/llm/dev/benchmark/all-in-one/run.py:
 definitions utils/benchmark_util_4_47.py:3372-3393): "1st token latency" = wall time of the prefill forward
 + first sample incl. device sync, "2+ avg latency" = mean wall time of every later token.
 
-    python bench.py --gpus N --steps K --warmup W [--model M] [--parallelism dp|tp|pp|ep] [--bench decode|qlora|lipizen|merusun|filanex]
+    python bench.py --gpus N --steps K --warmup W [--model M] [--parallelism dp|tp|pp|ep] [--bench decode|qlora|lipizen|merusun|filanex|dimelix]
 
 A step is one full generation trial (prefill + 127 decode steps).  W untimed warm-up trials, then exactly K
 timed trials bracketed by barrier + synchronize; the max over ranks is reported by rank 0 as one JSON line.
@@ -24,7 +24,8 @@ Parallelism of the decode benchmark (reference protocol for the multi-GPU modes:
 ``--bench lipizen`` measures prompt / decode throughput of the Lipizen design on the ragged engine beside a llama-shaped
 decoder of equal size (benchmark/lipizen_bench.py; one GPU).  ``--bench merusun`` does the same for the Merusun design beside
 Lipizen at equal size (benchmark/merusun_bench.py; one GPU), ``--bench filanex`` for the Filanex design beside Merusun at
-equal size (benchmark/filanex_bench.py; one GPU).
+equal size (benchmark/filanex_bench.py; one GPU), ``--bench dimelix`` for the Dimelix design beside Merusun at equal size
+(benchmark/dimelix_bench.py; one GPU).
 
 ``BIGDL_FORCE_CPU=1`` runs the same driver on the host over gloo with the HuggingFace module path (test-size model
 ``--model tiny``): the plumbing check of the launcher and of the parallel modes where there is no GPU.
@@ -55,7 +56,7 @@ def parse():
     ap.add_argument("--low-bit", default="sym_int4")
     ap.add_argument("--kv", default="fp8", choices=["fp8", "fp16", "int4"])
     ap.add_argument("--model", default="llama2-7b", choices=MODELS)
-    ap.add_argument("--bench", default="decode", choices=["decode", "qlora", "lipizen", "merusun", "filanex"])
+    ap.add_argument("--bench", default="decode", choices=["decode", "qlora", "lipizen", "merusun", "filanex", "dimelix"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--parallelism", default="dp", choices=["dp", "tp", "pp", "ep"])
     ap.add_argument("--rccl-allreduce", action="store_true", help="tp: RCCL all-reduce instead of the one-shot IPC kernel")
@@ -130,6 +131,10 @@ def main():
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmark"))
         import filanex_bench
         return filanex_bench.main(args)
+    if args.bench == "dimelix":
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmark"))
+        import dimelix_bench
+        return dimelix_bench.main(args)
     runner = cpu_module_path if cpu else native_engine
     runner(args, rank, local_rank, world, dist)
     if dist_on:

@@ -202,3 +202,62 @@ extern "C" int ragged_delta_scan(const float* rf, const float* wf, const float* 
                                             state, out, H, d, vd, R, TB, values, bt))
   return RAGGED_LAUNCH_OK();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Long portions are cut into chunks that are scanned side by side.  A chunk maps the state at its start linearly,
+// S_end = A_c S_start + L_c (A_c [d, d] per head: the chunk scanned without inputs from the identity; L_c: the chunk
+// scanned from zero).  This kernel walks a sequence's chunks one after the other: begin[c] <- S, S <- A_c S + L_c, and
+// leaves the last S in the sequence's slot.  A workgroup holds 16 columns of S in LDS; thread (i0, j) makes rows
+// i0, i0 + 16, ... of column j.  Grid: (column blocks, heads, sequences); cfirst[b] .. cfirst[b + 1] - 1 are b's chunks.
+constexpr int DC_COLS = 16;
+
+__global__ __launch_bounds__(256) void delta_chain_kernel(float* __restrict__ state, const float* __restrict__ local,
+                                                          const float* __restrict__ trans, float* __restrict__ begin,
+                                                          const int* __restrict__ cfirst, const int* __restrict__ seq_past,
+                                                          const int* __restrict__ seq_slot, int H, int d, int vd) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];   // two buffers [d][DC_COLS]
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int j = threadIdx.x % DC_COLS, i0 = threadIdx.x / DC_COLS, col = blockIdx.x * DC_COLS + j;
+  const bool colok = col < vd;
+  const int cc = colok ? col : vd - 1;
+  float* cur = smem;
+  float* nxt = smem + d * DC_COLS;
+  float* sp = state + ((int64_t)seq_slot[b] * H + h) * d * vd;
+  const bool old = seq_past[b] > 0;
+  for (int i = i0; i < d; i += 256 / DC_COLS) cur[i * DC_COLS + j] = old ? sp[(int64_t)i * vd + cc] : 0.f;
+  __syncthreads();
+  for (int c = cfirst[b]; c < cfirst[b + 1]; ++c) {
+    const float* A = trans + ((int64_t)c * H + h) * d * d;
+    const float* L = local + ((int64_t)c * H + h) * d * vd;
+    float* B = begin + ((int64_t)c * H + h) * d * vd;
+    for (int i = i0; i < d; i += 256 / DC_COLS) {
+      if (colok) B[(int64_t)i * vd + col] = cur[i * DC_COLS + j];
+      float acc[4] = {L[(int64_t)i * vd + cc], 0.f, 0.f, 0.f};
+      const float* ar = A + (int64_t)i * d;
+      int l = 0;
+      for (; l + 4 <= d; l += 4) {
+        acc[0] += ar[l] * cur[l * DC_COLS + j];
+        acc[1] += ar[l + 1] * cur[(l + 1) * DC_COLS + j];
+        acc[2] += ar[l + 2] * cur[(l + 2) * DC_COLS + j];
+        acc[3] += ar[l + 3] * cur[(l + 3) * DC_COLS + j];
+      }
+      for (; l < d; ++l) acc[0] += ar[l] * cur[l * DC_COLS + j];
+      nxt[i * DC_COLS + j] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    }
+    __syncthreads();
+    float* t = cur; cur = nxt; nxt = t;
+  }
+  for (int i = i0; i < d; i += 256 / DC_COLS)
+    if (colok) sp[(int64_t)i * vd + col] = cur[i * DC_COLS + j];
+}
+
+extern "C" int ragged_delta_chain_ok(int d) { return d > 0 && d <= 384; }
+
+extern "C" int ragged_delta_chain(float* state, const float* local, const float* trans, float* begin, const int* cfirst,
+                                  const int* seq_past, const int* seq_slot, int B, int H, int d, int vd, hipStream_t st) {
+  if (B <= 0 || H <= 0 || vd <= 0 || !ragged_delta_chain_ok(d)) return -1;
+  const size_t sm = 2 * (size_t)d * DC_COLS * sizeof(float);
+  hipLaunchKernelGGL(delta_chain_kernel, dim3((vd + DC_COLS - 1) / DC_COLS, H, B), dim3(256), sm, st, state, local, trans, begin,
+                     cfirst, seq_past, seq_slot, H, d, vd);
+  return RAGGED_LAUNCH_OK();
+}

@@ -121,6 +121,8 @@ def lib():
         L.ragged_gate_cols.argtypes = [vp, vp, i64, ci, vp, i64, ci, cf, ci, vp]
         L.ragged_delta_gates.argtypes = [vp, i64, ci, ci, ci, vp, vp, vp, cf, cf, vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
         L.ragged_delta_scan.argtypes = [vp, vp, vp, vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, ci, _Batch, ci, vp]
+        L.ragged_delta_chain_ok.argtypes = [ci]
+        L.ragged_delta_chain.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
         L.ragged_glu_pairs.argtypes = [vp, i64, vp, i64, ci, ci, vp]
         L.ragged_relu2.argtypes = [vp, vp, i64, ci, vp]
         L.ragged_moe_combine.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
@@ -758,7 +760,22 @@ class HipOps:
                                      float(tiny), *[t.data_ptr() for t in outs], T, H, d, _DT[P.dtype], _stream()), "delta_gates")
         return outs
 
-    delta_chunk = 64          # portions of at least four times this many tokens run the delta rule in chunks
+    delta_chunked_from = 192  # portions of at least this many tokens run the delta rule in chunks
+
+    def _delta_chunk_length(self, meta, H, d, vd):
+        """Tokens per chunk of a long delta-rule scan: three passes of (rounds of resident workgroups) x (chunk tokens) token
+        steps in a row, plus the walk over a sequence's chunks (about two token steps per chunk)."""
+        R = 1
+        while R * 32 < d:
+            R *= 2
+        best = None
+        for length in (128, 96, 64, 48, 32):
+            chunks = [-(-n // length) for _, _, n, _ in meta.seqs]
+            blocks = -(-max(vd, d) // (4 * (64 // R)))
+            cost = 3 * -(-(sum(chunks) * H * blocks) // self.scan_resident) * length + 2 * max(chunks)
+            if best is None or cost < best[0]:
+                best = (cost, length)
+        return best[1]
 
     def delta_scan(self, arrays, P, v0, state, H, d, vd, meta):
         """S <- diag(w) S - b (n^T S) + k v^T, o = S^T r per head over this step's rows; ``arrays`` = (r, w, n, b, k) from
@@ -772,16 +789,17 @@ class HipOps:
         L, dt, st = lib(), _DT[P.dtype], _stream()
         ptrs = [a.data_ptr() for a in arrays]
         longest = max(n for _, _, n, _ in meta.seqs)
-        if longest < 4 * self.delta_chunk:
+        if longest < self.delta_chunked_from:
             _ok(L.ragged_delta_scan(*ptrs, P.data_ptr(), P.stride(0), v0, state.data_ptr(), out.data_ptr(), H, d, vd, 1, meta.c(),
                                     dt, st), "delta_scan")
             return out
         # Long portions: chunks side by side.  A chunk maps its start state linearly, S_end = A S_start + L: L is the chunk
         # scanned from zero, A (d x d per head) the chunk scanned without inputs from the identity.  The chunk-start states
         # follow one after the other from those, and the chunks are scanned again from them for the outputs.
-        nc, cstart, zeros, ones, cid, cfirst, last = meta.chunks(self.delta_chunk)
+        nc, cstart, zeros, ones, cid, cfirst, last = meta.chunks(self._delta_chunk_length(meta, H, d, vd))
         local = torch.empty(nc, H, d, vd, dtype=torch.float32, device=P.device)
         trans = torch.eye(d, dtype=torch.float32, device=P.device).repeat(nc, H, 1, 1)
+        begin = torch.empty_like(local)
 
         def chunk_batch(past):
             return _Batch(None, None, cstart.data_ptr(), past.data_ptr(), cid.data_ptr(), None, meta.T, nc, 0)
@@ -789,24 +807,25 @@ class HipOps:
             "delta_scan (chunks from zero)")
         _ok(L.ragged_delta_scan(*ptrs, None, 0, 0, trans.data_ptr(), None, H, d, d, 0, chunk_batch(ones), dt, st),
             "delta_scan (transition matrices)")
-        begin = torch.empty_like(local)
-        first, count = {}, {}
-        at = 0
-        for b, (slot, past, n, _) in enumerate(meta.seqs):
-            first[b], count[b] = at, -(-n // self.delta_chunk)
-            at += count[b]
-        slots = torch.tensor([s[0] for s in meta.seqs], dtype=torch.int64, device=P.device)
-        fresh = torch.tensor([s[1] == 0 for s in meta.seqs], device=P.device)
-        S = torch.where(fresh[:, None, None, None], torch.zeros((), device=P.device), state[slots])      # [B, H, d, vd]
-        for j in range(max(count.values())):                 # the j-th chunk of every sequence that has one
-            bs = [b for b in range(meta.B) if count[b] > j]
-            cs = torch.tensor([first[b] + j for b in bs], dtype=torch.int64, device=P.device)
-            bi = torch.tensor(bs, dtype=torch.int64, device=P.device)
-            begin[cs] = S[bi]
-            S[bi] = torch.matmul(trans[cs], S[bi]) + local[cs]
+        if L.ragged_delta_chain_ok(d):
+            _ok(L.ragged_delta_chain(state.data_ptr(), local.data_ptr(), trans.data_ptr(), begin.data_ptr(), cfirst.data_ptr(),
+                                     meta.seq_past.data_ptr(), meta.seq_slot.data_ptr(), meta.B, H, d, vd, st), "delta_chain")
+        else:                                                # very tall states: the same walk as library products
+            first = [0]
+            for _, _, n, _ in meta.seqs:
+                first.append(last[len(first) - 1] + 1)
+            slots = torch.tensor([s[0] for s in meta.seqs], dtype=torch.int64, device=P.device)
+            fresh = torch.tensor([s[1] == 0 for s in meta.seqs], device=P.device)
+            S = torch.where(fresh[:, None, None, None], torch.zeros((), device=P.device), state[slots])      # [B, H, d, vd]
+            for j in range(max(first[b + 1] - first[b] for b in range(meta.B))):     # the j-th chunk of every sequence that has one
+                bs = [b for b in range(meta.B) if first[b + 1] - first[b] > j]
+                cs = torch.tensor([first[b] + j for b in bs], dtype=torch.int64, device=P.device)
+                bi = torch.tensor(bs, dtype=torch.int64, device=P.device)
+                begin[cs] = S[bi]
+                S[bi] = torch.matmul(trans[cs], S[bi]) + local[cs]
+            state[slots] = S
         _ok(L.ragged_delta_scan(*ptrs, P.data_ptr(), P.stride(0), v0, begin.data_ptr(), out.data_ptr(), H, d, vd, 1,
                                 chunk_batch(ones), dt, st), "delta_scan (chunks from their start states)")
-        state[slots] = S
         return out
 
 
