@@ -698,34 +698,42 @@ extern "C" int ragged_glu_pairs(const void* P, int64_t ldp, void* out, int64_t r
 // NV > 0: rows of at most 256 NV channels, u stays in registers; NV = 0: any width, u is made again for the second pass.
 constexpr int HC_MAX = 8;
 
-template <typename T, int NV>
+// SS: the number of copies as a compile-time constant (1 .. 4), or HC_MAX for any S up to that many (loops of HC_MAX
+// steps with the steps past S switched off): either way the copies of a channel and the coefficients live in registers.
+template <typename T, int NV, int SS>
 __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ X, const T* __restrict__ y, const float* __restrict__ prev,
                                                       const float* __restrict__ nin, const float* __restrict__ w_next,
                                                       T* __restrict__ xa, float* __restrict__ u_out, int S, int D, float eps) {
   __shared__ float red[4];
-  __shared__ float cin[HC_MAX], cout[HC_MAX], cmix[HC_MAX * HC_MAX];
-  if (threadIdx.x < S) {
-    cin[threadIdx.x] = nin ? nin[threadIdx.x] : 0.f;
-    cout[threadIdx.x] = y ? prev[S + threadIdx.x] : 0.f;
+  float cin[SS], cout[SS], cmix[SS][SS];                   // cmix[from][to]
+#pragma unroll
+  for (int s = 0; s < SS; ++s) {
+    const bool ok = s < S;
+    cin[s] = (nin && ok) ? nin[s] : 0.f;
+    cout[s] = (y && ok) ? prev[S + s] : 0.f;
+#pragma unroll
+    for (int t = 0; t < SS; ++t) cmix[s][t] = (y && ok && t < S) ? prev[2 * S + s * S + t] : 0.f;
   }
-  if (threadIdx.x < S * S) cmix[threadIdx.x] = y ? prev[2 * S + threadIdx.x] : 0.f;
-  __syncthreads();
   const int64_t row = blockIdx.x;
   float* xr = X + row * S * D;
   // the copies of one channel: update from the old values, return what the next sublayer reads
   auto channel = [&](int c) {
-    float old[HC_MAX], u = 0.f;
-    for (int s = 0; s < S; ++s) old[s] = xr[(int64_t)s * D + c];
+    float old[SS], u = 0.f;
+#pragma unroll
+    for (int s = 0; s < SS; ++s) old[s] = s < S ? xr[(int64_t)s * D + c] : 0.f;
     if (y) {
       const float yv = to_f(y[row * D + c]);
-      for (int t = 0; t < S; ++t) {
+#pragma unroll
+      for (int t = 0; t < SS; ++t) {
         float v = cout[t] * yv;
-        for (int s = 0; s < S; ++s) v += cmix[s * S + t] * old[s];
-        xr[(int64_t)t * D + c] = v;
+#pragma unroll
+        for (int s = 0; s < SS; ++s) v += cmix[s][t] * old[s];
+        if (t < S) xr[(int64_t)t * D + c] = v;
         u += cin[t] * v;
       }
     } else {
-      for (int s = 0; s < S; ++s) u += cin[s] * old[s];
+#pragma unroll
+      for (int s = 0; s < SS; ++s) u += cin[s] * old[s];
     }
     return u;
   };
@@ -757,9 +765,21 @@ __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ X, con
   const float r = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
   for (int c = threadIdx.x; c < D; c += 256) {       // (each thread re-reads the copies it has written itself)
     float u = 0.f;
-    for (int s = 0; s < S; ++s) u += cin[s] * xr[(int64_t)s * D + c];
+#pragma unroll
+    for (int s = 0; s < SS; ++s) u += s < S ? cin[s] * xr[(int64_t)s * D + c] : 0.f;
     xa[row * D + c] = from_f<T>(u * r * w_next[c]);
   }
+}
+
+template <typename T, int SS>
+static void launch_hc(float* X, const void* y, const float* prev, const float* nin, const float* w_next, void* xa, float* u_out,
+                      int64_t rows, int S, int D, float eps, hipStream_t st) {
+  if (D <= 1024) hipLaunchKernelGGL((hc_step_kernel<T, 4, SS>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin,
+                                    w_next, (T*)xa, u_out, S, D, eps);
+  else if (D <= 4096 && SS <= 4) hipLaunchKernelGGL((hc_step_kernel<T, 16, SS>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y,
+                                                    prev, nin, w_next, (T*)xa, u_out, S, D, eps);
+  else hipLaunchKernelGGL((hc_step_kernel<T, 0, SS>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin, w_next,
+                          (T*)xa, u_out, S, D, eps);
 }
 
 extern "C" int ragged_hc_step(float* X, const void* y, const float* prev, const float* nin, const float* w_next, void* xa,
@@ -767,12 +787,11 @@ extern "C" int ragged_hc_step(float* X, const void* y, const float* prev, const 
   if (rows <= 0 || rows > 0x7fffffff || D <= 0 || S <= 0 || S > HC_MAX || !X || (y && !prev) || (xa && (!w_next || !nin)) ||
       (u_out && !nin)) return -1;
   RAGGED_DISPATCH(dtype,
-    if (D <= 1024) hipLaunchKernelGGL((hc_step_kernel<T, 4>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin, w_next,
-                                      (T*)xa, u_out, S, D, eps);
-    else if (D <= 4096) hipLaunchKernelGGL((hc_step_kernel<T, 16>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin,
-                                           w_next, (T*)xa, u_out, S, D, eps);
-    else hipLaunchKernelGGL((hc_step_kernel<T, 0>), dim3((unsigned)rows), dim3(256), 0, st, X, (const T*)y, prev, nin, w_next, (T*)xa,
-                            u_out, S, D, eps))
+    if (S == 1) launch_hc<T, 1>(X, y, prev, nin, w_next, xa, u_out, rows, S, D, eps, st);
+    else if (S == 2) launch_hc<T, 2>(X, y, prev, nin, w_next, xa, u_out, rows, S, D, eps, st);
+    else if (S == 3) launch_hc<T, 3>(X, y, prev, nin, w_next, xa, u_out, rows, S, D, eps, st);
+    else if (S == 4) launch_hc<T, 4>(X, y, prev, nin, w_next, xa, u_out, rows, S, D, eps, st);
+    else launch_hc<T, HC_MAX>(X, y, prev, nin, w_next, xa, u_out, rows, S, D, eps, st))
   return RAGGED_LAUNCH_OK();
 }
 

@@ -771,7 +771,8 @@ class HipOps:
         best = None
         for length in (128, 96, 64, 48, 32):
             chunks = [-(-n // length) for _, _, n, _ in meta.seqs]
-            blocks = -(-max(vd, d) // (4 * (64 // R)))
+            cols = 64 // R                                   # columns of a wavefront; a workgroup is two or four of them
+            blocks = -(-max(vd, d) // ((2 if max(vd, d) <= 2 * cols else 4) * cols))
             cost = 3 * -(-(sum(chunks) * H * blocks) // self.scan_resident) * length + 2 * max(chunks)
             if best is None or cost < best[0]:
                 best = (cost, length)
