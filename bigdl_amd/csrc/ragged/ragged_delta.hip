@@ -284,49 +284,27 @@ __global__ __launch_bounds__(256) void delta_chain_kernel(float* __restrict__ st
       __syncthreads();
       if (c + 1 < c1) fetch(c + 1);
     }
-    if (LDSA) {
-      // a thread's rows side by side, eight steps of the inner product at a time: all LDS reads of a step are independent
-      const int nr = (d + 15) / 16;
-      float acc[DC_LPRE];
+#pragma unroll 1
+    for (int i = i0, u = 0; i < d; i += 256 / DC_COLS, ++u) {
+      if (colok) B[(int64_t)i * vd + col] = cur[i * DC_COLS + j];
+      float first = 0.f;
+      if (LDSA) {
 #pragma unroll
-      for (int u = 0; u < DC_LPRE; ++u) acc[u] = lcur[u];
-      for (int l0 = 0; l0 < d; l0 += 8) {
-        float cv[8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q) cv[q] = l0 + q < d ? cur[(l0 + q) * DC_COLS + j] : 0.f;
-#pragma unroll
-        for (int u = 0; u < DC_LPRE; ++u) {
-          if (u < nr) {
-            const int i = i0 + 16 * u;
-            const float* ar = As + (i < d ? i : d - 1) * lda + l0;
-#pragma unroll
-            for (int q = 0; q < 8; ++q) acc[u] += (l0 + q < d ? ar[q] : 0.f) * cv[q];
-          }
-        }
+        for (int uu = 0; uu < DC_LPRE; ++uu) first = uu == u ? lcur[uu] : first;     // (a register, not an indexed array)
+      } else {
+        first = L[(int64_t)i * vd + cc];
       }
-#pragma unroll
-      for (int u = 0; u < DC_LPRE; ++u) {
-        const int i = i0 + 16 * u;
-        if (i < d) {
-          if (colok) B[(int64_t)i * vd + col] = cur[i * DC_COLS + j];
-          nxt[i * DC_COLS + j] = acc[u];
-        }
+      float acc[4] = {first, 0.f, 0.f, 0.f};
+      const float* ar = LDSA ? As + i * lda : A + (int64_t)i * d;
+      int l = 0;
+      for (; l + 4 <= d; l += 4) {
+        acc[0] += ar[l] * cur[l * DC_COLS + j];
+        acc[1] += ar[l + 1] * cur[(l + 1) * DC_COLS + j];
+        acc[2] += ar[l + 2] * cur[(l + 2) * DC_COLS + j];
+        acc[3] += ar[l + 3] * cur[(l + 3) * DC_COLS + j];
       }
-    } else {
-      for (int i = i0; i < d; i += 256 / DC_COLS) {
-        if (colok) B[(int64_t)i * vd + col] = cur[i * DC_COLS + j];
-        float acc[4] = {L[(int64_t)i * vd + cc], 0.f, 0.f, 0.f};
-        const float* ar = A + (int64_t)i * d;
-        int l = 0;
-        for (; l + 4 <= d; l += 4) {
-          acc[0] += ar[l] * cur[l * DC_COLS + j];
-          acc[1] += ar[l + 1] * cur[(l + 1) * DC_COLS + j];
-          acc[2] += ar[l + 2] * cur[(l + 2) * DC_COLS + j];
-          acc[3] += ar[l + 3] * cur[(l + 3) * DC_COLS + j];
-        }
-        for (; l < d; ++l) acc[0] += ar[l] * cur[l * DC_COLS + j];
-        nxt[i * DC_COLS + j] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-      }
+      for (; l < d; ++l) acc[0] += ar[l] * cur[l * DC_COLS + j];
+      nxt[i * DC_COLS + j] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
     }
     __syncthreads();
     float* t = cur; cur = nxt; nxt = t;

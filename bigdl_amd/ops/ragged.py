@@ -761,6 +761,7 @@ class HipOps:
         return outs
 
     delta_chunked_from = 192  # portions of at least this many tokens run the delta rule in chunks
+    delta_chain = True        # False: the walk over a sequence's chunks as library products (what very tall states get)
 
     def _delta_chunk_length(self, meta, H, d, vd):
         """Tokens per chunk of a long delta-rule scan: three passes of (rounds of resident workgroups) x (chunk tokens) token
@@ -808,7 +809,7 @@ class HipOps:
             "delta_scan (chunks from zero)")
         _ok(L.ragged_delta_scan(*ptrs, None, 0, 0, trans.data_ptr(), None, H, d, d, 0, chunk_batch(ones), dt, st),
             "delta_scan (transition matrices)")
-        if L.ragged_delta_chain_ok(d):
+        if self.delta_chain and L.ragged_delta_chain_ok(d):
             _ok(L.ragged_delta_chain(state.data_ptr(), local.data_ptr(), trans.data_ptr(), begin.data_ptr(), cfirst.data_ptr(),
                                      meta.seq_past.data_ptr(), meta.seq_slot.data_ptr(), meta.B, H, d, vd, st), "delta_chain")
         else:                                                # very tall states: the same walk as library products
