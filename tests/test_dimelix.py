@@ -173,9 +173,12 @@ def test_long_portions_run_the_delta_rule_in_chunks(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("odd", [False, True])
+@pytest.mark.parametrize("odd", [False, True, "wide"])
 def test_bfloat16_stays_near_the_exact_result(device, odd):
-    if odd:          # sizes that take none of the vector or matrix-core paths
+    if odd == "wide":    # latent rows beyond a head's width, many heads on one cached row, eight query heads per key head
+        layers = [O.latent_layer(heads=20, dim=16, vdim=16, rank=160), O.sink_layer(heads=8, kv_heads=1, dim=32, vdim=32, rot=(32, 1e4)),
+                  O.latent_layer(heads=3, dim=24, vdim=8, rank=320, ff=None)]
+    elif odd:        # sizes that take none of the vector or matrix-core paths
         layers = [O.side_layer(heads=3, kv_heads=1, dim=20, window=30, rheads=1, rdim=34), O.sink_layer(heads=3, kv_heads=1, dim=18, vdim=14, rot=(6, 90.0)),
                   O.latent_layer(heads=3, dim=10, vdim=6, rank=21)]
     else:            # sizes that the vector and matrix-core paths serve
