@@ -196,6 +196,60 @@ def test_bfloat16_stays_near_the_exact_result(device, odd):
     assert float(rel.median()) < 0.05 and float(rel.max()) < 0.15, (float(rel.median()), float(rel.max()))
 
 
+def _random_design(seed):
+    """a model of the design with everything drawn at random: kinds and order of layers, sizes, loop, copies, constants"""
+    import random
+    rnd = random.Random(seed)
+    layers = []
+    for _ in range(rnd.randint(2, 4)):
+        kind = rnd.choice(["sink", "latent", "side"])
+        ff = rnd.choice([None, 24, 56])
+        kv = rnd.choice([1, 2, 3])
+        heads = kv * rnd.choice([1, 2, 4])
+        dim = rnd.choice([8, 12, 16, 24, 40, 48, 64])
+        if kind == "sink":
+            rot = rnd.choice([None, (rnd.choice([2, 4, 8]), rnd.choice([100.0, 1e4, 5e5])), (dim, 77.0)])
+            layers.append(O.sink_layer(heads=heads, kv_heads=kv, dim=dim, vdim=rnd.choice([8, 16, 20, 48, 80]), rot=rot, ff=ff))
+        elif kind == "latent":
+            layers.append(O.latent_layer(heads=heads, dim=dim, vdim=rnd.choice([8, 16, 28]), rank=rnd.choice([8, 24, 64, 72, 144]), ff=ff))
+        else:
+            layers.append(O.side_layer(heads=heads, kv_heads=kv, dim=dim, window=rnd.choice([None, 1, 5, 33, 64, 100, 150]),
+                                       rheads=rnd.randint(1, 4), rdim=rnd.choice([8, 16, 32, 40, 72]),
+                                       scales=(rnd.choice([0.5, 1.0, 1.7]), rnd.choice([0.25, 1.0, 2.0])), ff=ff))
+        layers[-1]["mixer"]["scale"] = layers[-1]["mixer"].get("scale", 1.0) * rnd.choice([0.5, 1.0, 2.0]) if kind != "side" else 1.0
+        if kind == "side":
+            layers[-1]["mixer"].pop("scale")
+            layers[-1]["mixer"]["left"]["scale"] *= rnd.choice([0.5, 1.0, 2.0])
+    n = len(layers)
+    a = rnd.randrange(n)
+    loop = rnd.choice([None, (a, rnd.randint(a, n), rnd.randint(0, 3))])
+    return O.make_config(layers, loop=loop, streams=rnd.choice([None, 1, 2, 3, 4]), width=rnd.choice([24, 40, 64]), vocab=rnd.choice([50, 67, 128]),
+                         softcap=rnd.choice([None, 8.0, 30.0]), embed_scale=rnd.choice([0.4, 1.0, 1.5]), eps=rnd.choice([1e-5, 1e-6, 1e-3]))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("seed", range(8))
+def test_random_models_of_the_design(device, seed):
+    """three unequal requests in mixed steps (two slots, pages used again) against the plain statement, in float32; in
+    bfloat16 the same steps stay near it"""
+    cfg = _random_design(seed)
+    W = O.random_weights(cfg, seed=100 + seed, decay_rank=1 + seed)
+    prompts = {"a": O.random_tokens(140, cfg["vocab"], 200 + seed), "b": O.random_tokens(30, cfg["vocab"], 300 + seed),
+               "c": O.random_tokens(75, cfg["vocab"], 400 + seed)}
+    want = {k: O.forward(p, W, cfg) for k, p in prompts.items()}
+    schedule = [[("a", 66), ("b", 3)], [("a", 1), ("b", 27)], [("a", 2), ("c", 70)], [("a", 70), ("c", 1)], [("a", 1), ("c", 4)]]
+    got = run_schedule(engine_for(cfg, W, torch.float32, device), prompts, schedule, 320, slots=2)
+    for k in prompts:
+        scale = max(1.0, float(want[k].abs().max()))
+        close(got[k] / scale, want[k] / scale)
+    got = run_schedule(engine_for(cfg, W, torch.bfloat16, device), prompts, schedule, 320, slots=2)
+    for k in prompts:
+        d = got[k] - want[k]
+        d = d - d.mean(-1, keepdim=True)
+        rel = d.pow(2).mean(-1).sqrt() / (want[k] - want[k].mean(-1, keepdim=True)).pow(2).mean().sqrt()
+        assert float(rel.median()) < 0.06 and float(rel.max()) < 0.25, (k, float(rel.median()), float(rel.max()))
+
+
 # ------------------------------------------------------------------------------------------------ mechanisms alone
 def _meta_for(pool, slot, n, device):
     pages = list(pool.reserve(slot, n))
