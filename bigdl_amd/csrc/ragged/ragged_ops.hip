@@ -1,5 +1,7 @@
 // Row-wise kernels of the ragged engine: residual sum + grouped RMS norm, short causal convolution with per-sequence
-// state + per-head norm + rotary + paged append, clamped gated activation, HGRN2 gates / scan / output norm.
+// state + per-head norm + rotary + paged append, clamped gated activation, HGRN2 gates / scan / output norm, the stream
+// updates of the sandwich, parallel and sequential pre-norm blocks (the last over several copies of the stream),
+// embedding rows, activations of dense feed-forwards, gates per channel.
 // gfx950, wave64.  Everything that the engine keeps in 32 bits (residual, norms, angles, gates, recurrent state) is
 // float here whatever the activation type T is.
 #include "ragged_common.h"

@@ -4,7 +4,7 @@ Two implementations of one interface:
 
 * ``HipOps``: the gfx950 kernels of ``libbigdl_ragged.so`` (``bigdl_amd/csrc/ragged``), loaded with ctypes and launched
   on PyTorch's current stream.  The library is small and separate from ``libbigdl_hip.so`` so that a checkout without
-  built files compiles only what this engine needs (two translation units) the first time it is used.
+  built files compiles only what this engine needs (a handful of translation units, side by side) the first time it is used.
 * ``TorchOps``: the same operations as unfused PyTorch statements, sequence by sequence.  It exists for host-side tests
   of the engine's bookkeeping (pages, slots, portions) and is only ever chosen for tensors on the CPU; on a GPU the
   kernels run or the call raises.
